@@ -26,6 +26,20 @@ from tokenmill_amd.cache.allocator import OutOfPages, PageAllocator, SlotAllocat
 RELEASED = -1       # a block-table entry whose page the window has passed
 
 
+@dataclass(frozen=True)
+class _WindowOnly:
+    """A group described by its window alone."""
+    window: int | None
+    chunk = None
+
+    @property
+    def keeps_all(self) -> bool:
+        return self.window is None
+
+    def first_needed(self, num_computed: int) -> int:
+        return 0 if self.window is None else max(0, num_computed - self.window + 1)
+
+
 class AllocStatus(enum.Enum):
     OK = 0
     LATER = 1       # not enough free pages now
@@ -46,13 +60,16 @@ class RequestCache:
 
 
 class CacheManager:
-    def __init__(self, group_windows: list[int | None], num_pages: int | list[int], page_size: int,
+    def __init__(self, group_windows: list, num_pages: int | list[int], page_size: int,
                  num_state_slots: int, watermark: float = 0.0):
+        """``group_windows``: per group its window (None: every token is kept), or the group's ``KVCacheSpec``
+        (``CachePools.group_specs``), which may also say that keys before the current chunk are never read again."""
         if page_size < 1:
             raise ValueError("page_size must be at least 1")
         self.page_size = page_size
-        self.windows = list(group_windows)
-        self.any_window = any(w is not None for w in self.windows)
+        self.specs = [w if hasattr(w, "first_needed") else _WindowOnly(w) for w in group_windows]
+        self.windows = [s.window for s in self.specs]
+        self.any_window = any(not s.keeps_all for s in self.specs)
         counts = [num_pages] * len(self.windows) if isinstance(num_pages, int) else list(num_pages)
         if len(counts) != len(self.windows):
             raise ValueError("one page count per group")
@@ -139,16 +156,17 @@ class CacheManager:
         return True
 
     def release_behind_window(self, rc: RequestCache, num_computed: int) -> int:
-        """Give back, in windowed groups, the pages that no later token can see: with
-        ``num_computed`` tokens cached, the next query sits at position >= num_computed and sees
-        keys from num_computed - W + 1 on. Returns the number of pages given back."""
+        """Give back, in groups that keep a window or only the current chunk, the pages that no later token
+        can see: with ``num_computed`` tokens cached, the next query sits at position >= num_computed and sees
+        keys from num_computed - W + 1 on, and none from before the start of the chunk that holds position
+        num_computed. Returns the number of pages given back."""
         given = 0
         if not self.any_window:
             return given
-        for g, window in enumerate(self.windows):
-            if window is None:
+        for g, spec in enumerate(self.specs):
+            if spec.keeps_all:
                 continue
-            first_needed = max(0, num_computed - window + 1)
+            first_needed = spec.first_needed(num_computed)
             upto = min(first_needed // self.page_size, len(rc.tables[g]))
             table = rc.tables[g]
             back = [table[i] for i in range(rc.released[g], upto) if table[i] != RELEASED]

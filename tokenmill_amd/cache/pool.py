@@ -2,8 +2,8 @@
 
 Per group two tensors in the model's storage type: keys [cache layers of the group, pages,
 page_size, kv_heads, head_dim], the reference's layout (reference
-src/infer/kv/paged_cache.py:1-6,28-34), and values [cache layers, pages, kv_heads, head_dim,
-page_size]: inside a page the values lie key-contiguous for each (head, d), which is the operand
+src/infer/kv/paged_cache.py:1-6,28-34), and values [cache layers, pages, kv_heads, value size,
+page_size] (the value size is the head size unless a group's spec says otherwise): inside a page the values lie key-contiguous for each (head, d), which is the operand
 layout of the MFMA attention kernels (no transposition through LDS). Per state-holding layer one
 tensor [slots, *shape].
 """
@@ -40,7 +40,7 @@ class CachePools:
                 members[g].append(j)
         self.k = [torch.zeros((len(members[g]), counts[g], page_size, s.kv_heads, s.head_dim), dtype=dtype,
                               device=device) for g, s in enumerate(self.groups)]
-        self.v = [torch.zeros((len(members[g]), counts[g], s.kv_heads, s.head_dim, page_size), dtype=dtype,
+        self.v = [torch.zeros((len(members[g]), counts[g], s.kv_heads, s.value_dim, page_size), dtype=dtype,
                               device=device) for g, s in enumerate(self.groups)]
         self.states: dict[int, torch.Tensor] = {}
         views: list = [None] * len(specs)
@@ -67,6 +67,11 @@ class CachePools:
     def windows(self) -> list[int | None]:
         return [s.window for s in self.groups]
 
+    @property
+    def group_specs(self) -> list[KVCacheSpec]:
+        """What the cache manager needs to know of each group (which keys later tokens can still read)."""
+        return list(self.groups)
+
     def reset_state_slot(self, slot: int) -> None:
         for t in self.states.values():
             t[slot].zero_()
@@ -80,4 +85,4 @@ class CachePools:
     def bytes_per_token(model, dtype) -> int:
         """Cache bytes one token takes over all layers (reference src/infer/config.py:37-39)."""
         size = torch.empty((), dtype=dtype).element_size()
-        return sum(2 * s.kv_heads * s.head_dim * size for s in model.cache_specs() if isinstance(s, KVCacheSpec))
+        return sum(s.kv_heads * (s.head_dim + s.value_dim) * size for s in model.cache_specs() if isinstance(s, KVCacheSpec))

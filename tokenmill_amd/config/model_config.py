@@ -141,6 +141,101 @@ class Qwen2Config:
         return d
 
 
+@dataclass(frozen=True)
+class ModinexLayer:
+    """One entry of a Modinex model's list of layers."""
+    type: str                                  # "attention" | "gla"
+    mixer: dict                                # the mixer's sizes and constants, as config.json gives them
+    ff: int | None                             # width of the dense feed-forward; None: the layer has none
+
+
+@dataclass(frozen=True)
+class ModinexConfig:
+    """The Modinex decoder: token embedding plus a learned position table; layers that each name their mixer
+    (sigmoid attention in chunks, or gated linear attention) and may have a dense feed-forward; a norm in groups
+    before and behind every sublayer. Every size and constant that can differ between two models of the design is
+    read here from config.json; sizes it does not give (the width of the narrow projection in front of a gla
+    mixer's decays) come from the checkpoint's tensors."""
+
+    vocab_size: int
+    hidden_size: int
+    max_position_embeddings: int
+    norm_eps: float
+    norm_groups: int
+    layers: tuple[ModinexLayer, ...]
+    eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
+
+    architecture = "Modinex"
+    MIXERS = ("attention", "gla")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, raw: dict, generation: dict | None = None) -> "ModinexConfig":
+        norm = _require(raw, "norm")
+        layers = []
+        for i, entry in enumerate(_require(raw, "layers")):
+            kind = entry.get("type")
+            if kind not in cls.MIXERS:
+                raise ConfigError(f"layers[{i}]: type '{kind}' is not one of {list(cls.MIXERS)}")
+            mixer = entry.get("mixer")
+            if not isinstance(mixer, dict):
+                raise ConfigError(f"layers[{i}] has no 'mixer' sizes")
+            mlp = entry.get("mlp")
+            if mlp is not None:
+                if mlp.get("kind", "dense") != "dense":
+                    raise ConfigError(f"layers[{i}]: feed-forward kind '{mlp.get('kind')}' is not supported (dense only)")
+                if "ff" not in mlp:
+                    raise ConfigError(f"layers[{i}]: the feed-forward has no 'ff' width")
+            need = ("heads", "dim", "vdim") + (("scale",) if kind == "attention" else ("tau",))
+            for key in need:
+                if mixer.get(key) is None:
+                    raise ConfigError(f"layers[{i}]: the {kind} mixer has no '{key}'")
+            layers.append(ModinexLayer(kind, dict(mixer), int(mlp["ff"]) if mlp is not None else None))
+        cfg = cls(vocab_size=int(_require(raw, "vocab")), hidden_size=int(_require(raw, "width")),
+                  max_position_embeddings=int(_require(raw, "max_positions")), norm_eps=float(_require(norm, "eps")),
+                  norm_groups=int(norm.get("groups", 1)), layers=tuple(layers),
+                  eos_token_ids=collect_eos_ids(([generation] if generation else []) + [raw]))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        for name in ("vocab_size", "hidden_size", "max_position_embeddings", "norm_groups"):
+            if getattr(self, name) <= 0:
+                raise ConfigError(f"{name} must be positive, got {getattr(self, name)}")
+        if self.hidden_size % self.norm_groups:
+            raise ConfigError(f"norm.groups {self.norm_groups} does not divide the width {self.hidden_size}")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if not self.layers:
+            raise ConfigError("a model needs at least one layer")
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            for key in ("heads", "dim", "vdim"):
+                if int(m[key]) <= 0:
+                    raise ConfigError(f"layers[{i}]: {key} must be positive")
+            if layer.type == "attention":
+                kv = int(m.get("kv_heads") or m["heads"])
+                if kv <= 0 or int(m["heads"]) % kv:
+                    raise ConfigError(f"layers[{i}]: {m['heads']} heads do not divide into {kv} kv heads")
+                rot = m.get("rot")
+                if rot:
+                    dims = int(rot.get("dims", 0))
+                    if dims < 0 or dims % 2 or dims > int(m["dim"]):
+                        raise ConfigError(f"layers[{i}]: rot.dims {dims} must be even and at most dim {m['dim']}")
+                    if dims and not float(rot.get("base", 0)) > 0:
+                        raise ConfigError(f"layers[{i}]: rot.base must be positive")
+                mask = m.get("mask")
+                if mask and mask.get("size") is not None and int(mask["size"]) <= 0:
+                    raise ConfigError(f"layers[{i}]: mask.size must be positive")
+            elif not float(m["tau"]) > 0:
+                raise ConfigError(f"layers[{i}]: tau must be positive")
+            if layer.ff is not None and layer.ff <= 0:
+                raise ConfigError(f"layers[{i}]: ff must be positive")
+
+
 def read_json(path: Path) -> dict:
     try:
         return json.loads(path.read_text())

@@ -45,9 +45,11 @@ def get_architecture(name: str) -> Architecture:
 
 def architecture_name(raw: dict) -> str:
     archs = raw.get("architectures")
-    if not archs or not isinstance(archs, list):
-        raise ConfigError("config.json has no 'architectures' list to choose the model by")
-    return str(archs[0])
+    if archs and isinstance(archs, list):
+        return str(archs[0])
+    if isinstance(raw.get("architecture"), str):         # some writers name the one architecture directly
+        return raw["architecture"]
+    raise ConfigError("config.json has no 'architectures' list (or 'architecture' name) to choose the model by")
 
 
 def load_config(model_dir: str | Path):

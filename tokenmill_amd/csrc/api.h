@@ -118,6 +118,37 @@ int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int out_stride, 
                         const void* v_pool, const int* block_tables, int table_width, const int* tiles, int n_tiles,
                         int H, int KVH, int D, int page, float scale, int window, hipStream_t stream);
 
+// out[t] = table[ids[t]] + places[positions[t]] as 32-bit rows (a learned position table beside the token table).
+int tm_embed_gather_pos(const void* table, const void* places, int dtype, const int* ids, const int* positions,
+                        float* out, int T, int hidden, int vocab, int max_pos, hipStream_t stream);
+
+int tm_gelu_tanh(const void* in, void* out, int dtype, long long n, hipStream_t stream);
+
+// RMS norm in `groups` equal consecutive parts of a row, around a sublayer (norm_groups.hip):
+// resid[r] += norm(y[r]; post_w) (post_w null: y as it is; y null: nothing), out[r] = norm(resid[r]; pre_w) (out null: none).
+int tm_group_norm(float* resid, const void* y, const void* post_w, const int* rows, const void* pre_w, int w_dtype,
+                  void* out, int dtype, int R, int hidden, int groups, float eps, hipStream_t stream);
+
+// Attention with sigmoid weights that are not normalized over the keys, keys of size D and values of size Dv, within
+// chunks and / or a window (attention_sigmoid.hip). qkv rows = [H x D | G x D | G x Dv]; q_w, k_w: weights [D] of the
+// per-head RMS norm of q and k (both null: none); head_bias [H] is added to the scaled score (null: none).
+int tm_qk_norm_rope_store(void* qkv, int ld, int dtype, int T, int H, int G, int D, int Dv, int rot, const float* q_w,
+                          const float* k_w, float eps, const float* cos_t, const float* sin_t, const int* positions,
+                          const int* slots, void* k_pool, void* v_pool, int page, int write_kv, hipStream_t stream);
+int tm_attn_sigmoid_paged(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+                          const int* block_tables, int table_width, const int* seq_of_token, const int* positions,
+                          const float* head_bias, int T, int H, int G, int D, int Dv, int page, float scale, int chunk,
+                          int window, int dtype, hipStream_t stream);
+
+// Gated linear attention (gla.hip): the decays from the gate projection, the recurrence over a step's rows request by
+// request with the state [slots, H, D, Dv] in 32-bit, and the per-head norm of the result times silu(gate).
+int tm_gla_decay(const float* z, float* a, float tau, long long n, hipStream_t stream);
+int tm_gla_scan(const void* proj, int ld, int q_off, int k_off, int v_off, int dtype, const float* decay, float* o,
+                float* state, const int* cu_q_lens, const int* state_slots, int S, int H, int D, int Dv, float q_scale,
+                hipStream_t stream);
+int tm_gla_out_gate(const float* o, const void* gate, int ldg, int dtype, const float* w, void* y, int T, int H, int Dv,
+                    float eps, hipStream_t stream);
+
 int tm_argmax_work_chunks(int V);
 int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);
 

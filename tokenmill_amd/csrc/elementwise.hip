@@ -35,6 +35,40 @@ extern "C" int tm_embed_gather(const void* table, int dtype, const int* ids, flo
 }
 
 // ------------------------------------------------------------------------------------------
+// embedding rows plus learned position rows -> 32-bit residual stream: out[t] = table[ids[t]] + places[positions[t]]
+// (the sum in 32-bit; no scaling of either)
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_gather_pos_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                        const T* __restrict__ places, const int* __restrict__ positions,
+                                        float* __restrict__ out, int hidden, int vocab, int max_pos) {
+    const int t = blockIdx.x;
+    int id = ids[t], p = positions[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);       // the host rejects such ids and positions; never read outside
+    p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);
+    const T* row = table + (size_t)id * hidden;
+    const T* prow = places + (size_t)p * hidden;
+    float* o = out + (size_t)t * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) o[c] = Elem<T>::load(row + c) + Elem<T>::load(prow + c);
+}
+
+extern "C" int tm_embed_gather_pos(const void* table, const void* places, int dtype, const int* ids, const int* positions,
+                                   float* out, int T, int hidden, int vocab, int max_pos, hipStream_t stream) {
+    if (T <= 0) return TM_OK;
+    if (hidden <= 0 || vocab <= 0 || max_pos <= 0 || !places || !positions) return TM_ERR_ARG;
+    if (dtype == TM_F32)
+        embed_gather_pos_kernel<float><<<T, 256, 0, stream>>>((const float*)table, ids, (const float*)places, positions, out,
+                                                             hidden, vocab, max_pos);
+    else if (dtype == TM_BF16)
+        embed_gather_pos_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)table, ids, (const bf16_t*)places, positions,
+                                                              out, hidden, vocab, max_pos);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// ------------------------------------------------------------------------------------------
 // residual += delta ; out = weight * round(residual * rsqrt(mean(residual^2) + eps))
 //                                                    (reference src/infer/model/layers.py:41-44,
 //                                                     src/infer/model/qwen2.py:22-23)
@@ -377,6 +411,56 @@ extern "C" int tm_silu_mul(const void* gu, void* out, int dtype, int T, int I, h
         silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
     else if (dtype == TM_BF16)
         silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// out[i] = gelu_tanh(in[i]) = 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), computed in 32-bit (in place allowed)
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_tanh_f32(float z) {
+    const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+    return 0.5f * z * (1.f + tanhf(u));
+}
+
+template <typename T>
+__global__ void gelu_tanh_kernel(const T* __restrict__ in, T* __restrict__ out, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        Elem<T>::store(out + i, gelu_tanh_f32(Elem<T>::load(in + i)));
+}
+
+// bfloat16, eight elements (16 bytes) per thread and step
+__global__ void gelu_tanh_bf16x8_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, size_t groups) {
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < groups; idx += (size_t)gridDim.x * blockDim.x) {
+        const uint4 v = *(const uint4*)(in + 8 * idx);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float a = gelu_tanh_f32(__uint_as_float(w[k] << 16)), b = gelu_tanh_f32(__uint_as_float(w[k] & 0xffff0000u));
+            o[k] = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+        }
+        *(uint4*)(out + 8 * idx) = uint4{o[0], o[1], o[2], o[3]};
+    }
+}
+
+extern "C" int tm_gelu_tanh(const void* in, void* out, int dtype, long long n, hipStream_t stream) {
+    if (n <= 0) return TM_OK;
+    if (!in || !out) return TM_ERR_ARG;
+    if (dtype == TM_BF16 && n % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0) {
+        const size_t groups = (size_t)n / 8, want = (groups + 255) / 256;
+        gelu_tanh_bf16x8_kernel<<<(int)(want < 65536 ? want : 65536), 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, groups);
+        TM_CHECK_LAUNCH();
+        return TM_OK;
+    }
+    const size_t want = ((size_t)n + 255) / 256;
+    const int blocks = (int)(want < 16384 ? want : 16384);
+    if (dtype == TM_F32)
+        gelu_tanh_kernel<float><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, (size_t)n);
+    else if (dtype == TM_BF16)
+        gelu_tanh_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, (size_t)n);
     else
         return TM_ERR_ARG;
     TM_CHECK_LAUNCH();

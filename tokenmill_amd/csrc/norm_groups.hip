@@ -1,0 +1,109 @@
+// RMS norm in groups, around a sublayer: the result y of a mixer or feed-forward is normed, added to the 32-bit
+// residual stream, and the sum is normed again for the sublayer that follows, in one kernel.
+//
+//   norm_g(v)[c] = w[c] * v[c] / sqrt(mean(v[group of c]^2) + eps)     the row cut into `groups` equal consecutive parts
+//
+//   resid[r] += norm_g(y[r]; post_w)     (post_w == nullptr: y is added as it is; y == nullptr: nothing is added)
+//   out[r]    = norm_g(resid[r]; pre_w)  (out == nullptr: no second norm)
+//
+// rows == nullptr: every row, the residual updated in place. rows != nullptr: row rows[r] is read, nothing is written
+// back, out row r (the rows whose logits are wanted).
+//
+// Everything is 32-bit; a bfloat16 result is rounded once, where it is stored. The sums of squares have one order
+// per (width, groups): a group (or, with fewer than four groups, each of its 4 / groups equal pieces) is summed by
+// one wavefront, lanes striding over it, and a group's pieces are added in their order.
+#include "common.h"
+#include "api.h"
+
+#define GN_THREADS 256
+#define GN_WAVES (GN_THREADS / TM_WAVE)
+
+// sums of squares of the units of a row held in `v` (LDS or global), into part[units]
+template <typename Load>
+__device__ __forceinline__ void unit_sums(Load at, float* part, int glen, int split, int units) {
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    const int plen = (glen + split - 1) / split;
+    for (int u = wave; u < units; u += GN_WAVES) {
+        const int g = u / split, i = u - g * split;
+        const int lo = g * glen + i * plen;
+        const int hi = min(lo + plen, (g + 1) * glen);
+        float ss = 0.f;
+        for (int c = lo + lane; c < hi; c += TM_WAVE) {
+            const float x = at(c);
+            ss += x * x;
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) part[u] = ss;
+    }
+}
+
+__device__ __forceinline__ float group_scale(const float* part, int g, int split, int glen, float eps) {
+    float ss = part[g * split];
+    for (int i = 1; i < split; ++i) ss += part[g * split + i];
+    return 1.0f / sqrtf(ss / (float)glen + eps);
+}
+
+template <typename T, typename WT>
+__global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(float* __restrict__ resid, const T* __restrict__ y,
+                                                                const WT* __restrict__ post_w,
+                                                                const int* __restrict__ rows,
+                                                                const WT* __restrict__ pre_w, T* __restrict__ out,
+                                                                int hidden, int groups, int split, float eps) {
+    extern __shared__ float lds[];
+    float* xs = lds;                    // the row, [hidden]
+    float* part = lds + hidden;         // [groups * split]
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* x = resid + src * hidden;
+    const int glen = hidden / groups, units = groups * split;
+    for (int c = threadIdx.x; c < hidden; c += GN_THREADS) xs[c] = x[c];
+    if (y) {
+        const T* yr = y + src * hidden;
+        if (post_w) {
+            unit_sums([&](int c) { return Elem<T>::load(yr + c); }, part, glen, split, units);
+            __syncthreads();
+        }
+        for (int c = threadIdx.x; c < hidden; c += GN_THREADS) {
+            float d = Elem<T>::load(yr + c);
+            if (post_w) d = Elem<WT>::load(post_w + c) * (d * group_scale(part, c / glen, split, glen, eps));
+            const float v = xs[c] + d;
+            xs[c] = v;
+            if (!rows) x[c] = v;
+        }
+    }
+    if (!out) return;
+    __syncthreads();
+    unit_sums([&](int c) { return xs[c]; }, part, glen, split, units);
+    __syncthreads();
+    T* o = out + (size_t)r * hidden;
+    for (int c = threadIdx.x; c < hidden; c += GN_THREADS)
+        Elem<T>::store(o + c, Elem<WT>::load(pre_w + c) * (xs[c] * group_scale(part, c / glen, split, glen, eps)));
+}
+
+extern "C" int tm_group_norm(float* resid, const void* y, const void* post_w, const int* rows, const void* pre_w,
+                             int w_dtype, void* out, int dtype, int R, int hidden, int groups, float eps,
+                             hipStream_t stream) {
+    if (R <= 0) return TM_OK;
+    if (hidden <= 0 || groups <= 0 || hidden % groups || !(eps > 0.f) || !resid) return TM_ERR_ARG;
+    if ((out == nullptr) != (pre_w == nullptr)) return TM_ERR_ARG;
+    if (!y && post_w) return TM_ERR_ARG;
+    const int split = groups >= GN_WAVES ? 1 : GN_WAVES / groups;
+    const size_t lds = ((size_t)hidden + (size_t)groups * split) * sizeof(float);
+    if (lds > 64 * 1024) return TM_ERR_ARG;
+    if (dtype == TM_F32 && w_dtype == TM_F32)
+        group_norm_kernel<float, float><<<R, GN_THREADS, lds, stream>>>(resid, (const float*)y, (const float*)post_w, rows,
+                                                                       (const float*)pre_w, (float*)out, hidden, groups,
+                                                                       split, eps);
+    else if (dtype == TM_BF16 && w_dtype == TM_BF16)
+        group_norm_kernel<bf16_t, bf16_t><<<R, GN_THREADS, lds, stream>>>(resid, (const bf16_t*)y, (const bf16_t*)post_w,
+                                                                         rows, (const bf16_t*)pre_w, (bf16_t*)out, hidden,
+                                                                         groups, split, eps);
+    else if (dtype == TM_BF16 && w_dtype == TM_F32)
+        group_norm_kernel<bf16_t, float><<<R, GN_THREADS, lds, stream>>>(resid, (const bf16_t*)y, (const float*)post_w, rows,
+                                                                        (const float*)pre_w, (bf16_t*)out, hidden, groups,
+                                                                        split, eps);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}

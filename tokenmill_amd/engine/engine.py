@@ -62,7 +62,7 @@ class LLMEngine:
         self.eos_ids = set(getattr(model.config, "eos_token_ids", ()) or ())
         pages = num_cache_pages(cfg, model, self.dtype, self.device)
         self.pools = CachePools(model, pages, cfg.block_size, cfg.max_num_seqs, self.dtype, self.device)
-        self.cache = CacheManager(self.pools.windows, pages, cfg.block_size, cfg.max_num_seqs, cfg.watermark)
+        self.cache = CacheManager(self.pools.group_specs, pages, cfg.block_size, cfg.max_num_seqs, cfg.watermark)
         # timing the library's algorithms is this engine's choice: it travels with the engine's own step program
         tune = (TUNE_CANDIDATES, cfg.tune_gemm_every) if cfg.tune_gemm else None
         self.runner = ModelRunner(model, self.pools, max_positions=cfg.max_model_len, tune=tune)

@@ -160,7 +160,7 @@ class DecodeGraphs:
             slots = host[bk.g_slot[g][0]:bk.g_slot[g][1]]
             tabs = host[bk.g_tab[g][0]:bk.g_tab[g][1]].reshape(B, W)
             slots[:] = -1
-            windowed = runner.pools.groups[g].window is not None
+            windowed = not runner.pools.groups[g].keeps_all
             rows = bk.rows_held[g]
             new_slots = []
             for i, e in enumerate(entries):

@@ -64,16 +64,17 @@ def load_random_model(config: dict, seed: int, dtype: torch.dtype, device: torch
     g = torch.Generator(device=device).manual_seed(seed)
     tensors = {}
     for name, spec in sorted(model.tensor_specs().items()):
+        shape = spec.drawn_shape()
         if spec.kind == "int":
-            t = torch.arange(int(torch.tensor(spec.shape).prod()), dtype=torch.int32, device=device).reshape(spec.shape)
+            t = torch.arange(int(torch.tensor(shape).prod()), dtype=torch.int32, device=device).reshape(shape)
         elif spec.init == "ones":
-            t = torch.ones(spec.shape, dtype=torch.float32, device=device)
+            t = torch.ones(shape, dtype=torch.float32, device=device)
             if norm_std:
-                t += torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * norm_std
+                t += torch.randn(shape, generator=g, dtype=torch.float32, device=device) * norm_std
         elif spec.init == "zeros":
-            t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
+            t = torch.zeros(shape, dtype=torch.float32, device=device)
         else:
-            t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * std
+            t = torch.randn(shape, generator=g, dtype=torch.float32, device=device) * std
         tensors[name] = t if spec.kind == "int" else t.to(storage_dtype(torch.bfloat16, spec.kind, dtype))
     model.load(tensors, dtype, device, pack_weights=pack_weights)
     return model

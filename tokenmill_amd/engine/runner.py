@@ -211,7 +211,7 @@ class ModelRunner:
             slots_state[s0:s0 + n1] = [e.cache.state_slot for e in singles]
             for g in range(n_groups):
                 tabs = g_tab[g][0][s0 * W:(s0 + n1) * W].reshape(n1, W)
-                windowed = self.pools.groups[g].window is not None
+                windowed = not self.pools.groups[g].keeps_all
                 new_slots = []
                 for j, (e, p) in enumerate(zip(singles, p1)):
                     table = e.cache.tables[g]

@@ -23,7 +23,7 @@ def largest_step_bytes(cfg: EngineConfig, model, dtype, device) -> tuple[int, in
     lengths = [longest] * (n // longest) + ([n % longest] if n % longest else [])
     pages = sum(-(-s // cfg.block_size) for s in lengths)
     pools = CachePools(model, pages, cfg.block_size, len(lengths), dtype, device)
-    manager = CacheManager(pools.windows, pages, cfg.block_size, len(lengths))
+    manager = CacheManager(pools.group_specs, pages, cfg.block_size, len(lengths))
     runner = ModelRunner(model, pools, max_positions=cfg.max_model_len)
     torch.cuda.synchronize(device)
     before = torch.cuda.memory_allocated(device)          # weights and the throw-away pool

@@ -979,3 +979,205 @@ def argmax_rows_static(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _need(logits.device.index == torch.cuda.current_device(), "argmax (static): the logits' GPU must be the current device")
     _check(lib.tm_argmax_rows_static(_p(logits), c_int(R), c_int(V), _p(out), _stream()), "argmax_rows_static")
     return out
+
+
+# -------------------------------------------------------------------------------------------- learned positions, gelu
+
+def embed_gather_pos(table: torch.Tensor, places: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor,
+                     out: torch.Tensor) -> torch.Tensor:
+    """out[t] = table[ids[t]] + places[positions[t]] as 32-bit rows. table [V, hidden] and places [P, hidden] of one
+    type, ids and positions int32 [T], out float32 [T, hidden]."""
+    _gpu(table, places, ids, positions, out)
+    T = ids.numel()
+    V, hidden = table.shape
+    _need(table.is_contiguous() and places.is_contiguous() and out.is_contiguous(), "embed_gather_pos: operands must be contiguous")
+    _need(places.dim() == 2 and places.shape[1] == hidden and places.dtype == table.dtype,
+          f"embed_gather_pos: the position table must be [positions, {hidden}] of the token table's type")
+    _need(out.dtype == torch.float32 and tuple(out.shape) == (T, hidden), "embed_gather_pos: out must be float32 [T, hidden]")
+    _ints(ids, T, "ids")
+    _ints(positions, T, "positions")
+    _check(library().tm_embed_gather_pos(_p(table), _p(places), code(table.dtype), _p(ids), _p(positions), _p(out), c_int(T),
+                                         c_int(hidden), c_int(V), c_int(places.shape[0]), _stream()), "embed_gather_pos")
+    return out
+
+
+def gelu_tanh(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))), computed in 32-bit; ``out`` may be ``x``."""
+    _gpu(x, out)
+    _need(x.is_contiguous() and out.is_contiguous() and x.shape == out.shape and x.dtype == out.dtype,
+          "gelu_tanh: x and out must be contiguous, of one shape and type")
+    _check(library().tm_gelu_tanh(_p(x), _p(out), code(x.dtype), c_longlong(x.numel()), _stream()), "gelu_tanh")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- norm in groups
+
+GROUP_NORM_MAX_FLOATS = 16384 - 64        # what a row and its group sums may take of a block's 64 KiB of LDS
+
+
+def group_norm(resid: torch.Tensor, y: torch.Tensor | None, post_w: torch.Tensor | None, pre_w: torch.Tensor | None,
+               out: torch.Tensor | None, groups: int, eps: float, rows: torch.Tensor | None = None) -> torch.Tensor | None:
+    """RMS norm in ``groups`` equal consecutive parts of a row, around a sublayer:
+    resid += norm(y; post_w) (``post_w`` None: y as it is; ``y`` None: nothing is added), then
+    out = norm(resid; pre_w) (``out`` None: no second norm). With ``rows``: only those rows, out row r from resid row
+    rows[r], and resid is not written. resid float32 [T, hidden]; y, out of the model's type; weights [hidden]."""
+    _gpu(resid, y, post_w, pre_w, out, rows)
+    T, hidden = resid.shape
+    R = T if rows is None else rows.numel()
+    _need(resid.dtype == torch.float32 and resid.is_contiguous(), "group_norm: the residual stream is contiguous float32")
+    _need(groups >= 1 and hidden % groups == 0, f"group_norm: {groups} groups do not divide the width {hidden}")
+    _need(hidden + 4 * groups <= GROUP_NORM_MAX_FLOATS, f"group_norm: a row of {hidden} does not fit the kernel's LDS")
+    _need((out is None) == (pre_w is None), "group_norm: out and its norm's weight come together")
+    _need(post_w is None or y is not None, "group_norm: a norm of y needs y")
+    dtype = out.dtype if out is not None else y.dtype if y is not None else None
+    _need(dtype is not None, "group_norm: nothing to do")
+    if y is not None:
+        _need(y.dtype == dtype and tuple(y.shape) == (T, hidden) and y.is_contiguous(), f"group_norm: y must be {dtype} [{T}, {hidden}]")
+    if out is not None:
+        _need(tuple(out.shape) == (R, hidden) and out.is_contiguous(), f"group_norm: out must be [{R}, {hidden}]")
+    w_dtype = None
+    for w in (post_w, pre_w):
+        if w is not None:
+            _need(tuple(w.shape) == (hidden,) and w.is_contiguous(), "group_norm: a weight must be [hidden]")
+            _need(w_dtype in (None, w.dtype), "group_norm: both weights share one type")
+            w_dtype = w.dtype
+    _need(w_dtype is None or dtype == torch.bfloat16 or w_dtype == torch.float32, "group_norm: a float32 result needs float32 weights")
+    if rows is not None:
+        _ints(rows, R, "rows")
+    _need(eps > 0, "group_norm: eps must be positive")
+    _check(library().tm_group_norm(_p(resid), _p(y), _p(post_w), _p(rows), _p(pre_w), c_int(code(w_dtype or dtype)), _p(out),
+                                   c_int(code(dtype)), c_int(R), c_int(hidden), c_int(groups), c_float(eps), _stream()),
+           "group_norm")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- sigmoid attention
+
+def _check_pools_kv(k_pool: torch.Tensor, v_pool: torch.Tensor, G: int, D: int, Dv: int, dtype, who: str) -> int:
+    """K pool [pages, page, G, D], V pool [pages, G, Dv, page]; returns the page size."""
+    _need(k_pool.dim() == 4 and v_pool.dim() == 4 and k_pool.is_contiguous() and v_pool.is_contiguous(),
+          f"{who}: the cache pools must be contiguous 4-d tensors")
+    pages, page = k_pool.shape[0], k_pool.shape[1]
+    _need(tuple(k_pool.shape) == (pages, page, G, D), f"{who}: k_pool must be [pages, page, {G}, {D}]")
+    _need(tuple(v_pool.shape) == (pages, G, Dv, page), f"{who}: v_pool must be [pages, {G}, {Dv}, page]")
+    _need(k_pool.dtype == dtype and v_pool.dtype == dtype, f"{who}: the cache pools must have the type {dtype}")
+    return page
+
+
+def qk_norm_rope_store(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, q_w: torch.Tensor | None, k_w: torch.Tensor | None,
+                       eps: float, cos: torch.Tensor | None, sin: torch.Tensor | None, positions: torch.Tensor | None,
+                       slots: torch.Tensor | None, k_pool: torch.Tensor | None, v_pool: torch.Tensor | None) -> None:
+    """In place on qkv [T, H*D + G*D + G*Dv]: every head of q and k is divided by its root mean square and multiplied by
+    q_w / k_w (float32 [D], shared by the heads; both None: no norm), then its first 2 * cos.shape[1] channels are
+    rotated by the token's position (cos/sin float32 [max_pos, rot/2]; None: no rotation); k and v go to the tokens'
+    cache slots (pools None: not stored; a slot < 0 is not stored)."""
+    _gpu(qkv, q_w, k_w, cos, sin, positions, slots, k_pool, v_pool)
+    T = qkv.shape[0]
+    width = (H + G) * D + G * Dv
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == width, f"qk_norm_rope_store: qkv must be [T, {width}]")
+    _need(0 < D <= 256 and 0 < Dv, "qk_norm_rope_store: head sizes up to 256")
+    _need((q_w is None) == (k_w is None), "qk_norm_rope_store: q and k are normed together or not at all")
+    for w in (q_w, k_w):
+        if w is not None:
+            _need(w.dtype == torch.float32 and tuple(w.shape) == (D,) and w.is_contiguous(), f"qk_norm_rope_store: norm weights are float32 [{D}]")
+    rot = 0
+    if cos is not None:
+        rot = 2 * cos.shape[1]
+        _need(sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
+              and cos.is_contiguous() and sin.is_contiguous() and rot <= D, "qk_norm_rope_store: cos/sin float32 [max_pos, rot/2], rot <= D")
+        _ints(positions, T, "positions")
+    write = k_pool is not None
+    page = 0
+    if write:
+        page = _check_pools_kv(k_pool, v_pool, G, D, Dv, qkv.dtype, "qk_norm_rope_store")
+        _ints(slots, T, "slots")
+    ld = qkv.stride(0) if T > 1 else max(width, qkv.stride(0))
+    _check(library().tm_qk_norm_rope_store(_p(qkv), c_int(ld), c_int(code(qkv.dtype)), c_int(T), c_int(H), c_int(G), c_int(D),
+                                           c_int(Dv), c_int(rot), _p(q_w), _p(k_w), c_float(eps), _p(cos), _p(sin),
+                                           _p(positions), _p(slots), _p(k_pool), _p(v_pool), c_int(page), c_int(1 if write else 0),
+                                           _stream()), "qk_norm_rope_store")
+
+
+def attn_sigmoid_paged(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                       block_tables: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
+                       head_bias: torch.Tensor | None, H: int, G: int, D: int, Dv: int, scale: float, chunk: int = 0,
+                       window: int = 0) -> torch.Tensor:
+    """out[t, h] = sum over visible keys j of sigmoid(scale * q[t, h] . k[j] + head_bias[h]) * v[j]: every token of the step
+    over its request's cache (its own key included), from the start of its chunk of ``chunk`` positions (0: from the
+    first) and at most ``window`` back (0: any). q [T, >= H*D] with unit inner stride, out [T, H*Dv]."""
+    _gpu(q, out, k_pool, v_pool, block_tables, seq_of_token, positions, head_bias)
+    T = q.shape[0]
+    _need(q.stride(1) == 1 and q.shape[1] >= H * D and out.is_contiguous() and tuple(out.shape) == (T, H * Dv),
+          f"attention(sigmoid): q [T, >={H * D}] unit inner stride, out contiguous [T, {H * Dv}]")
+    _need(q.dtype == out.dtype, "attention(sigmoid): q and out share one type")
+    _need(H % G == 0 and 0 < D <= 256 and 0 < Dv <= 256, "attention(sigmoid): head sizes up to 256, heads a multiple of kv heads")
+    page = _check_pools_kv(k_pool, v_pool, G, D, Dv, q.dtype, "attention(sigmoid)")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "attention(sigmoid): block_tables must be contiguous int32 [S, W]")
+    _ints(seq_of_token, T, "seq_of_token")
+    _ints(positions, T, "positions")
+    if head_bias is not None:
+        _need(head_bias.dtype == torch.float32 and tuple(head_bias.shape) == (H,) and head_bias.is_contiguous(),
+              f"attention(sigmoid): head_bias is float32 [{H}]")
+    _need(chunk >= 0 and window >= 0, "attention(sigmoid): chunk and window must be >= 0")
+    q_stride = q.stride(0) if T > 1 else max(q.stride(0), H * D)
+    _check(library().tm_attn_sigmoid_paged(_p(q), c_int(q_stride), _p(out), c_int(H * Dv), _p(k_pool), _p(v_pool), _p(block_tables),
+                                           c_int(block_tables.shape[1]), _p(seq_of_token), _p(positions), _p(head_bias), c_int(T),
+                                           c_int(H), c_int(G), c_int(D), c_int(Dv), c_int(page), c_float(scale), c_int(chunk),
+                                           c_int(window), c_int(code(q.dtype)), _stream()), "attn_sigmoid_paged")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- gated linear attention
+
+def gla_decay(z: torch.Tensor, tau: float, out: torch.Tensor | None = None) -> torch.Tensor:
+    """sigmoid(z)^(1/tau) as exp(logsigmoid(z) / tau), float32; in place unless ``out`` is given."""
+    out = z if out is None else out
+    _gpu(z, out)
+    _need(z.dtype == torch.float32 and out.dtype == torch.float32 and z.is_contiguous() and out.is_contiguous()
+          and z.shape == out.shape, "gla_decay: contiguous float32 tensors of one shape")
+    _need(tau > 0, "gla_decay: tau must be positive")
+    _check(library().tm_gla_decay(_p(z), _p(out), c_float(tau), c_longlong(z.numel()), _stream()), "gla_decay")
+    return out
+
+
+def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torch.Tensor, o: torch.Tensor, state: torch.Tensor,
+             cu_q_lens: torch.Tensor, state_slots: torch.Tensor, num_seqs: int, H: int, D: int, Dv: int, q_scale: float) -> torch.Tensor:
+    """The recurrence S = diag(decay_t) S + k_t v_t^T, o_t = S^T (q_scale * q_t) over the rows of each request of the
+    step in order, from and to the request's state row. proj [T, ld] holds q, k [H*D] and v [H*Dv] at the given column
+    offsets; decay float32 [T, H*D]; o float32 [T, H*Dv]; state float32 [slots, H, D, Dv]; cu_q_lens int32 [S+1];
+    state_slots int32 [S]."""
+    _gpu(proj, decay, o, state, cu_q_lens, state_slots)
+    T, ld_cols = proj.shape
+    _need(proj.stride(1) == 1, "gla_scan: proj rows have unit inner stride")
+    _need(0 < D <= 256 and Dv > 0 and H > 0, "gla_scan: key size up to 256")
+    for off, n in ((q_off, H * D), (k_off, H * D), (v_off, H * Dv)):
+        _need(0 <= off and off + n <= ld_cols, "gla_scan: q, k, v lie inside a row of proj")
+    _need(decay.dtype == torch.float32 and decay.is_contiguous() and tuple(decay.shape) == (T, H * D), f"gla_scan: decay float32 [{T}, {H * D}]")
+    _need(o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (T, H * Dv), f"gla_scan: o float32 [{T}, {H * Dv}]")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, D, Dv),
+          f"gla_scan: state float32 [slots, {H}, {D}, {Dv}]")
+    _ints(cu_q_lens, num_seqs + 1, "cu_q_lens")
+    _ints(state_slots, num_seqs, "state_slots")
+    _need(num_seqs <= 65535, "gla_scan: at most 65,535 requests a step")
+    ld = proj.stride(0) if T > 1 else max(ld_cols, proj.stride(0))
+    _check(library().tm_gla_scan(_p(proj), c_int(ld), c_int(q_off), c_int(k_off), c_int(v_off), c_int(code(proj.dtype)), _p(decay),
+                                 _p(o), _p(state), _p(cu_q_lens), _p(state_slots), c_int(num_seqs), c_int(H), c_int(D), c_int(Dv),
+                                 c_float(q_scale), _stream()), "gla_scan")
+    return o
+
+
+def gla_out_gate(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, y: torch.Tensor, H: int, Dv: int, eps: float) -> torch.Tensor:
+    """y[t, h] = w * o[t, h] / rms(o[t, h]) * silu(gate[t, h]). o float32 [T, H*Dv]; gate [T, >= H*Dv] (a view with unit
+    inner stride) and y [T, H*Dv] of the model's type; w float32 [Dv]."""
+    _gpu(o, gate, w, y)
+    T = o.shape[0]
+    _need(o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (T, H * Dv), f"gla_out_gate: o float32 [{T}, {H * Dv}]")
+    _need(gate.stride(1) == 1 and gate.shape[0] == T and gate.shape[1] >= H * Dv and gate.dtype == y.dtype, "gla_out_gate: gate [T, >= H*Dv] of y's type")
+    _need(y.is_contiguous() and tuple(y.shape) == (T, H * Dv), f"gla_out_gate: y [{T}, {H * Dv}]")
+    _need(w.dtype == torch.float32 and tuple(w.shape) == (Dv,) and w.is_contiguous(), f"gla_out_gate: w float32 [{Dv}]")
+    _need(eps > 0, "gla_out_gate: eps must be positive")
+    ldg = gate.stride(0) if T > 1 else max(gate.stride(0), H * Dv)
+    _check(library().tm_gla_out_gate(_p(o), _p(gate), c_int(ldg), c_int(code(y.dtype)), _p(w), _p(y), c_int(T), c_int(H), c_int(Dv),
+                                     c_float(eps), _stream()), "gla_out_gate")
+    return y

@@ -39,6 +39,15 @@ class Flow:
     x: torch.Tensor | None = None            # into a single operation: its input, already normed
     qkv: torch.Tensor | None = None          # into a single attention: q|k|v already projected, encoded and stored
     accumulate: bool = True                  # may an operation add its result into resid itself?
+    delta_norm: object | None = None         # a norm that delta passes before it is added (a block that norms its results)
+
+    def settle(self) -> None:
+        """Add a result that has to pass a norm on its way into the residual stream now: what comes next takes
+        only a plain pending result."""
+        if self.delta_norm is not None and self.delta is not None:
+            self.delta_norm.add_normed(self.resid, self.delta)
+            self.delta = None
+        self.delta_norm = None
 
 
 @dataclass
@@ -223,6 +232,7 @@ class StepProgram:
                 at_once: bool = False, _shared: dict | None = None) -> None:
         """Operations [first, first + count) as one call into the library. ``flow`` is updated in place: its delta
         becomes what the last operation left to be added (a view of this call's workspace) or None."""
+        flow.settle()
         T = step.num_tokens if step is not None else rows
         R = step.num_logit_rows if step is not None else 0
         nd = step.num_decode if step is not None else 0

@@ -85,7 +85,9 @@ class DecoderModel:
         emb, head, norm = self.embedding, self.head, self.final_norm
         if getattr(emb, "emit", lambda p: None)(program) is None:
             def embed(flow, step):
-                flow.resid, flow.delta = emb.forward(step.token_ids), None
+                # an embedding that adds something by position is handed the positions too
+                rows = emb.forward(step.token_ids, step.positions) if getattr(emb, "by_position", False) else emb.forward(step.token_ids)
+                flow.resid, flow.delta = rows, None
             program.foreign(emb, embed)
         for j, call in enumerate(self.run):
             self.layers[call.layer].emit(program, caches[j])
@@ -93,8 +95,11 @@ class DecoderModel:
             def logits(flow, step):
                 if step.num_logit_rows == 0:
                     flow.logits = torch.empty((0, head.vocab), dtype=torch.float32, device=flow.resid.device)
+                elif flow.delta_norm is not None and flow.delta is not None:
+                    flow.logits = head.forward(norm.add_norm(flow.resid, flow.delta, self.dtype, rows=step.logit_rows,
+                                                             delta_norm=flow.delta_norm))
                 else:
                     flow.logits = head.forward(norm.add_norm(flow.resid, flow.delta, self.dtype, rows=step.logit_rows))
-                flow.delta = None
+                flow.delta = flow.delta_norm = None
             program.foreign(head, logits)
         return program

@@ -22,10 +22,32 @@ from tokenmill_amd.weights.loader import TensorSpec
 
 @dataclass(frozen=True)
 class KVCacheSpec:
-    """Keys and values in pages. ``window``: None keeps every token; W keeps the last W."""
+    """Keys and values in pages. ``window``: None keeps every token; W keeps the last W. ``chunk``: C means that a
+    token never reads a key from before the start of its own chunk of C positions (counted from position 0), so the
+    pages of finished chunks can be given back. ``v_head_dim``: size of a value where it differs from a key's."""
     kv_heads: int
     head_dim: int
     window: int | None = None
+    v_head_dim: int | None = None
+    chunk: int | None = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_head_dim or self.head_dim
+
+    def first_needed(self, num_computed: int) -> int:
+        """With ``num_computed`` tokens cached, the next query sits at position num_computed or later: the first
+        position whose key it, or any later token, may still read."""
+        first = 0
+        if self.window is not None:
+            first = max(first, num_computed - self.window + 1)
+        if self.chunk is not None:
+            first = max(first, num_computed // self.chunk * self.chunk)
+        return first
+
+    @property
+    def keeps_all(self) -> bool:
+        return self.window is None and self.chunk is None
 
 
 @dataclass(frozen=True)
@@ -39,7 +61,7 @@ class StateSpec:
 class KVCacheView:
     """One cache layer as a mixer sees it."""
     k: torch.Tensor              # [pages, page_size, kv_heads, head_dim]
-    v: torch.Tensor              # [pages, kv_heads, head_dim, page_size]
+    v: torch.Tensor              # [pages, kv_heads, value size, page_size]
     group: int                   # index into StepContext.groups
     write: bool = True           # False: this layer reads a cache that another layer writes
 
@@ -122,6 +144,11 @@ class Norm(Part):
         follow it can compute themselves; None for any other norm."""
         return None
 
+    def add_normed(self, resid: torch.Tensor, y: torch.Tensor) -> None:
+        """resid (float32 [T, hidden]) += self(y), in place: this norm on a sublayer's result, on its way into the
+        residual stream. Only norms that stand behind a sublayer need it."""
+        raise NotImplementedError
+
 
 class NormedInput:
     """The input of a mixer or feed-forward that is still to be computed: norm(resid + delta).
@@ -130,8 +157,12 @@ class NormedInput:
     place) or, if it has a kernel that starts with the norm, takes ``fusable_rms()`` and reads
     ``resid`` itself. One of the two must happen, or a pending delta would be lost."""
 
-    def __init__(self, norm: Norm, resid: torch.Tensor, delta: torch.Tensor | None, dtype: torch.dtype):
+    def __init__(self, norm: Norm, resid: torch.Tensor, delta: torch.Tensor | None, dtype: torch.dtype,
+                 delta_norm: Norm | None = None):
+        """``delta_norm``: a norm that ``delta`` passes on its way into the residual stream (the block before
+        norms its sublayers' results); the norm that computes this input is then asked to do both."""
         self.norm, self.resid, self.delta, self.dtype = norm, resid, delta, dtype
+        self.delta_norm = delta_norm if delta is not None else None
         self._tensor: torch.Tensor | None = None
         self.taken = False                   # a kernel that starts at the norm has taken resid and delta as they are
 
@@ -141,8 +172,11 @@ class NormedInput:
 
     def tensor(self) -> torch.Tensor:
         if self._tensor is None:
-            self._tensor = self.norm.add_norm(self.resid, self.delta, self.dtype)
-            self.delta = None
+            if self.delta_norm is not None:
+                self._tensor = self.norm.add_norm(self.resid, self.delta, self.dtype, delta_norm=self.delta_norm)
+            else:
+                self._tensor = self.norm.add_norm(self.resid, self.delta, self.dtype)
+            self.delta = self.delta_norm = None
         return self._tensor
 
     def fusable_rms(self) -> tuple[torch.Tensor, float] | None:
@@ -154,7 +188,7 @@ class NormedInput:
     @property
     def lazy(self) -> bool:
         """Still to be computed, by a norm the kernel library computes itself?"""
-        return self._tensor is None and not self.taken and self.norm.rms_params() is not None
+        return self._tensor is None and not self.taken and self.delta_norm is None and self.norm.rms_params() is not None
 
     def take(self) -> tuple[torch.Tensor, torch.Tensor | None]:
         """(resid, delta) for an operation that adds and norms by itself; after this the input counts as computed."""
@@ -228,5 +262,6 @@ class Block(Part):
 
     def emit(self, program, cache) -> None:
         def run(flow, step):
+            flow.settle()
             flow.delta = self.forward(flow.resid, flow.delta, step, cache, program.dtype)
         program.foreign(self, run)

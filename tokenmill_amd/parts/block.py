@@ -41,12 +41,14 @@ class PreNormBlock(Block):
         operation for runs through its own ``forward`` between the library's operations."""
         if self.mixer.emit(program, self.norm_in, cache) is None:
             def mix(flow, step):
+                flow.settle()
                 x = NormedInput(self.norm_in, flow.resid, flow.delta, program.dtype)
                 flow.delta = self.mixer.forward(x, step, cache, residual=flow.resid)
                 assert x.delta is None, f"{type(self.mixer).__name__}.forward did not take its input"
             program.foreign(self.mixer, mix)
         if self.ffn.emit(program, self.norm_post) is None:
             def feed(flow, step):
+                flow.settle()
                 x = NormedInput(self.norm_post, flow.resid, flow.delta, program.dtype)
                 flow.delta = self.ffn.forward(x, step, residual=flow.resid)
                 assert x.delta is None, f"{type(self.ffn).__name__}.forward did not take its input"
@@ -58,3 +60,68 @@ class PreNormBlock(Block):
         feed-forward added its result itself)."""
         a = self.mixer.forward(NormedInput(self.norm_in, resid, delta, dtype), step, cache, residual=resid)
         return self.ffn.forward(NormedInput(self.norm_post, resid, a, dtype), step, residual=resid)
+
+
+class SandwichBlock(Block):
+    """A norm before and a norm behind each sublayer:
+
+        h = x + norm_mixed(mixer(norm_in(x)));   y = h + norm_fed(ffn(norm_post(h)))
+
+    A block without a feed-forward (``ffn`` None) has the first line only. The residual stream is the 32-bit tensor
+    every block updates in place. A sublayer's result is left pending together with the norm it has to pass
+    (``flow.delta``, ``flow.delta_norm``), so that the norm in front of the next sublayer, of this block or the
+    next, can norm it, add it and norm the sum in one kernel."""
+
+    def __init__(self, norm_in: Norm, mixer: Mixer, norm_mixed: Norm, norm_post: Norm | None = None,
+                 ffn: FeedForward | None = None, norm_fed: Norm | None = None,
+                 names: tuple[str, str, str, str, str, str] = ("norm1", "mix.", "norm1b", "norm2", "mlp.", "norm2b")):
+        if (ffn is None) != (norm_post is None) or (ffn is None) != (norm_fed is None):
+            raise ValueError("a feed-forward comes with the norm before it and the norm behind it, or not at all")
+        self.norm_in, self.mixer, self.norm_mixed = norm_in, mixer, norm_mixed
+        self.norm_post, self.ffn, self.norm_fed = norm_post, ffn, norm_fed
+        self.names = names
+
+    def _parts(self):
+        return [(p, n) for p, n in zip((self.norm_in, self.mixer, self.norm_mixed, self.norm_post, self.ffn, self.norm_fed),
+                                       self.names) if p is not None]
+
+    def tensor_specs(self, prefix: str):
+        specs = {}
+        for part, name in self._parts():
+            specs.update(part.tensor_specs(prefix + name))
+        return specs
+
+    def load(self, tensors, prefix: str) -> None:
+        for part, name in self._parts():
+            part.load(tensors, prefix + name)
+
+    def prepare(self, pack_weights: bool) -> None:
+        for part, _ in self._parts():
+            part.prepare(pack_weights)
+
+    def emit(self, program, cache) -> None:
+        """Each sublayer runs through its part's own ``forward``, between whatever operations of the kernel library
+        the model's other parts describe."""
+        def mix(flow, step):
+            x = NormedInput(self.norm_in, flow.resid, flow.delta, program.dtype, delta_norm=flow.delta_norm)
+            flow.delta, flow.delta_norm = self.mixer.forward(x, step, cache), self.norm_mixed
+            assert x.delta is None, f"{type(self.mixer).__name__}.forward did not take its input"
+        program.foreign(self.mixer, mix)
+        if self.ffn is not None:
+            def feed(flow, step):
+                x = NormedInput(self.norm_post, flow.resid, flow.delta, program.dtype, delta_norm=flow.delta_norm)
+                flow.delta, flow.delta_norm = self.ffn.forward(x, step), self.norm_fed
+                assert x.delta is None, f"{type(self.ffn).__name__}.forward did not take its input"
+            program.foreign(self.ffn, feed)
+
+    def forward(self, resid: torch.Tensor, delta: torch.Tensor | None, step: StepContext, cache,
+                dtype: torch.dtype) -> None:
+        """The block by itself: resid float32 [T, hidden] is updated in place with everything, ``delta`` (a plain
+        result of the block before, still to be added) included; nothing is left pending."""
+        y = self.mixer.forward(NormedInput(self.norm_in, resid, delta, dtype), step, cache)
+        if self.ffn is None:
+            self.norm_mixed.add_normed(resid, y)
+            return None
+        y = self.ffn.forward(NormedInput(self.norm_post, resid, y, dtype, delta_norm=self.norm_mixed), step)
+        self.norm_fed.add_normed(resid, y)
+        return None

@@ -10,37 +10,67 @@ from tokenmill_amd.parts.linear import Linear
 from tokenmill_amd.weights.loader import TensorSpec
 
 
-class TokenEmbedding(Part):
-    """x = E[ids], no scaling; rows are widened into the 32-bit residual stream."""
+class LearnedPositions(Part):
+    """A table with one learned row per position, added (unscaled) to the token's embedding row."""
 
-    def __init__(self, vocab: int, hidden: int, name: str = "weight"):
-        self.vocab, self.hidden, self.name = vocab, hidden, name
+    def __init__(self, max_positions: int, hidden: int, name: str = "weight"):
+        self.max_positions, self.hidden, self.name = max_positions, hidden, name
         self.weight: torch.Tensor | None = None
 
     def tensor_specs(self, prefix: str):
-        return {f"{prefix}{self.name}": TensorSpec((self.vocab, self.hidden))}
+        return {f"{prefix}{self.name}": TensorSpec((self.max_positions, self.hidden))}
 
     def load(self, tensors, prefix: str) -> None:
         self.weight = tensors[f"{prefix}{self.name}"]
 
+
+class TokenEmbedding(Part):
+    """x = E[ids], no scaling; rows are widened into the 32-bit residual stream. With ``places`` (a
+    ``LearnedPositions``) the row of the token's position is added, in 32-bit."""
+
+    def __init__(self, vocab: int, hidden: int, name: str = "weight", places: LearnedPositions | None = None):
+        self.vocab, self.hidden, self.name, self.places = vocab, hidden, name, places
+        self.weight: torch.Tensor | None = None
+
+    @property
+    def by_position(self) -> bool:
+        """Does ``forward`` need the tokens' positions beside their ids?"""
+        return self.places is not None
+
+    def tensor_specs(self, prefix: str):
+        specs = {f"{prefix}{self.name}": TensorSpec((self.vocab, self.hidden))}
+        if self.places is not None:
+            specs.update(self.places.tensor_specs(prefix))
+        return specs
+
+    def load(self, tensors, prefix: str) -> None:
+        self.weight = tensors[f"{prefix}{self.name}"]
+        if self.places is not None:
+            self.places.load(tensors, prefix)
+
     def emit(self, program) -> int | None:
+        if self.places is not None:
+            return None                         # the library's operation gathers token rows only
         return program.embedding(self, self.weight)
 
     def cost(self, label, step, rows):
-        return rows * self.hidden * (self.weight.element_size() + 4), 0
+        return rows * self.hidden * (self.weight.element_size() * (2 if self.places is not None else 1) + 4), 0
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, token_ids: torch.Tensor, positions: torch.Tensor | None = None) -> torch.Tensor:
         out = torch.empty((token_ids.numel(), self.hidden), dtype=torch.float32, device=token_ids.device)
         with profiling.label("embed", lambda: self.cost("embed", None, token_ids.numel())):
+            if self.places is not None:
+                return ops.embed_gather_pos(self.weight, self.places.weight, token_ids, positions, out)
             return ops.embed_gather(self.weight, token_ids, out)
 
 
 class OutputHead(Part):
     """logits = h W^T in 32-bit, W the embedding table itself when tied (no second copy)."""
 
-    def __init__(self, hidden: int, vocab: int, tied_to: TokenEmbedding | None, name: str = "lm_head"):
+    def __init__(self, hidden: int, vocab: int, tied_to: TokenEmbedding | None, name: str = "lm_head",
+                 suffixes: tuple[str, str] = (".weight", ".bias")):
         self.hidden, self.vocab, self.tied_to = hidden, vocab, tied_to
-        self.proj = Linear(hidden, vocab, name, bias=False, library_first=True)
+        self.proj = Linear(hidden, vocab, name, bias=False, library_first=True, suffixes=suffixes)
 
     def tensor_specs(self, prefix: str):
         return {} if self.tied_to is not None else self.proj.tensor_specs(prefix)

@@ -15,14 +15,16 @@ from tokenmill_amd.weights.loader import TensorSpec
 
 class Linear(Part):
     def __init__(self, in_features: int, out_features: list[int] | int, names: list[str] | str,
-                 bias: bool = False, library_first: bool = False):
+                 bias: bool = False, library_first: bool = False, suffixes: tuple[str, str] = (".weight", ".bias")):
         self.in_features = in_features
         self.out_splits = [out_features] if isinstance(out_features, int) else list(out_features)
         self.names = [names] if isinstance(names, str) else list(names)
         assert len(self.names) == len(self.out_splits)
         self.out_features = sum(self.out_splits)
         self.has_bias = bias
+        self.bias_init_zero = False
         self.library_first = library_first              # a wide matrix the library reads fastest at any row count
+        self.suffixes = suffixes                        # what a checkpoint appends to a name for the matrix and for the bias
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
         self.packed: ops.PackedWeight | None = None     # the matrix again in the order the decode kernels read
@@ -30,17 +32,19 @@ class Linear(Part):
 
     def tensor_specs(self, prefix: str) -> dict[str, TensorSpec]:
         specs = {}
+        sw, sb = self.suffixes
         for name, n in zip(self.names, self.out_splits):
-            specs[f"{prefix}{name}.weight"] = TensorSpec((n, self.in_features))
+            specs[f"{prefix}{name}{sw}"] = TensorSpec((n, self.in_features))
             if self.has_bias:
-                specs[f"{prefix}{name}.bias"] = TensorSpec((n,))
+                specs[f"{prefix}{name}{sb}"] = TensorSpec((n,), init="zeros" if self.bias_init_zero else "normal")
         return specs
 
     def load(self, tensors, prefix: str) -> None:
-        ws = [tensors[f"{prefix}{name}.weight"] for name in self.names]
+        sw, sb = self.suffixes
+        ws = [tensors[f"{prefix}{name}{sw}"] for name in self.names]
         self.weight = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0).contiguous()
         if self.has_bias:
-            bs = [tensors[f"{prefix}{name}.bias"] for name in self.names]
+            bs = [tensors[f"{prefix}{name}{sb}"] for name in self.names]
             self.bias = bs[0] if len(bs) == 1 else torch.cat(bs, dim=0).contiguous()
             if self.weight.dtype == torch.float32 and self.bias.dtype != torch.float32:
                 self.bias = self.bias.float()          # a 32-bit product adds a 32-bit bias

@@ -65,3 +65,37 @@ class SwiGLU(FeedForward):
         if x.shape[0] == 0:
             return None if residual is not None else torch.empty_like(x)
         return program.run_one(op, None, resid=residual, x=x.contiguous(), accumulate=residual is not None, rows=x.shape[0])
+
+
+class DenseFeedForward(FeedForward):
+    """down(act(up(x))) with one up matrix and no gate; ``activation``: "gelu_tanh", the tanh form of GELU,
+    0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), computed in 32-bit. Both products may have biases."""
+
+    ACTIVATIONS = {"gelu_tanh": ops.gelu_tanh}
+
+    def __init__(self, hidden: int, intermediate: int, activation: str = "gelu_tanh", bias: bool = True,
+                 names: tuple[str, str] = ("up", "down"), suffixes: tuple[str, str] = (".weight", ".bias")):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"activation '{activation}' is not one of {sorted(self.ACTIVATIONS)}")
+        self.hidden, self.intermediate, self.activation = hidden, intermediate, activation
+        self.up = Linear(hidden, intermediate, names[0], bias=bias, suffixes=suffixes)
+        self.down = Linear(intermediate, hidden, names[1], bias=bias, suffixes=suffixes)
+
+    def tensor_specs(self, prefix: str):
+        return {**self.up.tensor_specs(prefix), **self.down.tensor_specs(prefix)}
+
+    def load(self, tensors, prefix: str) -> None:
+        self.up.load(tensors, prefix)
+        self.down.load(tensors, prefix)
+
+    def cost(self, label: str, step: StepContext | None, rows: int) -> tuple[int, int]:
+        return self.up.cost(rows) if label == "gate_up" else self.down.cost(rows)
+
+    def forward(self, x, step: StepContext | None = None, residual: torch.Tensor | None = None):
+        from tokenmill_amd import profiling
+        x = as_tensor(x)
+        with profiling.label("gate_up", lambda: self.up.cost(x.shape[0])):
+            a = self.up.forward(x)
+            self.ACTIVATIONS[self.activation](a, a)
+        with profiling.label("down", lambda: self.down.cost(x.shape[0])):
+            return self.down.forward(a)

@@ -33,3 +33,51 @@ class RMSNorm(Norm):
 
     def rms_params(self):
         return self.weight, self.eps
+
+
+class GroupRMSNorm(Norm):
+    """RMS norm in groups: the row is cut into ``groups`` equal consecutive parts, each part is divided by its own
+    sqrt(mean(part^2) + eps), and the whole is multiplied by the weight; all of it in 32-bit, the result rounded
+    once. ``groups = 1`` is the usual RMS norm (rounded after the weight, not before it as ``RMSNorm`` does).
+
+    It can also stand behind a sublayer (``add_normed``: resid += self(y)); a ``GroupRMSNorm`` that is asked for
+    the next sublayer's input while such a result is pending does both in one kernel when the two agree on
+    groups and eps."""
+
+    def __init__(self, hidden: int, eps: float, groups: int = 1, name: str = "weight"):
+        if groups < 1 or hidden % groups:
+            raise ValueError(f"{groups} groups do not divide a width of {hidden}")
+        self.hidden, self.eps, self.groups, self.name = hidden, float(eps), groups, name
+        self.weight: torch.Tensor | None = None
+
+    def tensor_specs(self, prefix: str):
+        return {f"{prefix}{self.name}": TensorSpec((self.hidden,), init="ones")}
+
+    def load(self, tensors, prefix: str) -> None:
+        self.weight = tensors[f"{prefix}{self.name}"]
+
+    def _cost(self, n: int, out_bytes: int, added: int):
+        return n * self.hidden * (4 + out_bytes + added), 0
+
+    def add_norm(self, resid, delta, out_dtype, rows=None, delta_norm: Norm | None = None):
+        n = resid.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.hidden), dtype=out_dtype, device=resid.device)
+        post = None
+        if delta is not None and delta_norm is not None:
+            if isinstance(delta_norm, GroupRMSNorm) and (delta_norm.groups, delta_norm.eps) == (self.groups, self.eps):
+                post = delta_norm.weight
+            elif rows is None:
+                delta_norm.add_normed(resid, delta)
+                delta = None
+            else:
+                # only some rows are wanted and the residual is to stay as it is: the pending result's norm on a copy
+                resid = resid.index_select(0, rows.long())
+                delta_norm.add_normed(resid, delta.index_select(0, rows.long()))
+                delta, rows = None, None
+        added = 0 if delta is None else (4 if rows is None else 0) + delta.element_size()
+        with profiling.label("norm", lambda: self._cost(n, out.element_size(), added)):
+            return ops.group_norm(resid, delta, post, self.weight, out, self.groups, self.eps, rows)
+
+    def add_normed(self, resid, y) -> None:
+        with profiling.label("norm", lambda: self._cost(resid.shape[0], 4, y.element_size())):
+            ops.group_norm(resid, y, self.weight, None, None, self.groups, self.eps)

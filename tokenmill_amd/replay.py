@@ -51,7 +51,7 @@ class ReplaySession:
         # one page per request part empty beyond it
         self.num_pages = -(-max_tokens // page_size) + (0 if ROUND_TO % page_size == 0 else max_requests)
         self.pools = CachePools(self.model, self.num_pages, page_size, max_requests, dtype, device)
-        self.manager = CacheManager(self.pools.windows, self.num_pages, page_size, max_requests)
+        self.manager = CacheManager(self.pools.group_specs, self.num_pages, page_size, max_requests)
         self.runner = ModelRunner(self.model, self.pools, max_positions=max_positions)
         self.lengths: dict[str, int] = {}
 

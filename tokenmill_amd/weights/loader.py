@@ -22,10 +22,23 @@ from safetensors import safe_open
 
 @dataclass(frozen=True)
 class TensorSpec:
-    """One tensor a model expects in its checkpoint."""
-    shape: tuple[int, ...]
+    """One tensor a model expects in its checkpoint. A dimension given as None is the checkpoint's to decide (the
+    part reads it from the tensor it is handed); ``free`` holds the sizes such dimensions get, in their order,
+    when the tensor is drawn at random."""
+    shape: tuple[int | None, ...]
     kind: str = "float"          # "float" | "int"
     init: str = "normal"         # random-weights mode: "normal" | "ones" | "zeros" | "index"
+    free: tuple[int, ...] = ()
+
+    def fits(self, got: tuple[int, ...]) -> bool:
+        return len(got) == len(self.shape) and all(w is None or w == g for w, g in zip(self.shape, got))
+
+    def drawn_shape(self) -> tuple[int, ...]:
+        sizes = iter(self.free)
+        try:
+            return tuple(next(sizes) if n is None else n for n in self.shape)
+        except StopIteration:
+            raise ValueError(f"a tensor of shape {self.shape} has no size to be drawn with") from None
 
 
 class WeightsError(RuntimeError):
@@ -83,8 +96,8 @@ def read_checkpoint(model_dir, expected: dict[str, TensorSpec], dtype: torch.dty
                         unexpected.append(name)
                     continue
                 got = tuple(f.get_slice(name).get_shape())
-                if got != tuple(expected[name].shape):
-                    wrong.append((name, got, tuple(expected[name].shape)))
+                if not expected[name].fits(got):
+                    wrong.append((name, got, tuple("any" if n is None else n for n in expected[name].shape)))
                 where[name] = file
     missing = [n for n in expected if n not in where]
     if missing or unexpected or wrong:

@@ -32,18 +32,19 @@ def random_tensors(specs: dict[str, TensorSpec], seed: int, std: float = 0.02, n
     """(name, tensor) for every spec: "normal" ~ N(0, std); "ones" = 1 + N(0, norm_std)."""
     for name in sorted(specs):
         spec = specs[name]
+        shape = spec.drawn_shape()
         g = _generator(seed, name)
         if spec.kind == "int":
-            t = torch.arange(int(torch.tensor(spec.shape).prod()), dtype=torch.int32).reshape(spec.shape)
+            t = torch.arange(int(torch.tensor(shape).prod()), dtype=torch.int32).reshape(shape)
         elif spec.init == "ones":
-            t = torch.ones(spec.shape, dtype=torch.float32)
+            t = torch.ones(shape, dtype=torch.float32)
             if norm_std:
-                t += torch.randn(spec.shape, generator=g, dtype=torch.float32) * norm_std
+                t += torch.randn(shape, generator=g, dtype=torch.float32) * norm_std
             t = t.to(storage)
         elif spec.init == "zeros":
-            t = torch.zeros(spec.shape, dtype=storage)
+            t = torch.zeros(shape, dtype=storage)
         else:
-            t = (torch.randn(spec.shape, generator=g, dtype=torch.float32) * std).to(storage)
+            t = (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(storage)
         yield name, t
 
 
