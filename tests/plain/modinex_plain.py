@@ -124,7 +124,7 @@ def gla_recurrence(q, k, v, log_alpha, state=None):
 def gla_mixer(h, w, p, m, eps, dt, state=None, return_state: bool = False):
     T = h.shape[0]
     H, D, Dv = m["heads"], m["dim"], m["vdim"]
-    q = rnd(linear(h, w[p + "q"], None, dt) * D ** -0.5, dt).view(T, H, D)
+    q = (linear(h, w[p + "q"], None, dt) * D ** -0.5).view(T, H, D)
     k = linear(h, w[p + "k"], None, dt).view(T, H, D)
     v = linear(h, w[p + "v"], None, dt).view(T, H, Dv)
     z = linear(linear(h, w[p + "a1"], None, dt), w[p + "a2"], w[p + "a2.b"], dt, keep32=True).view(T, H, D)
@@ -145,7 +145,7 @@ def gelu_tanh(z):
 
 def dense_ff(h, w, p, dt):
     """down(gelu_tanh(up h + b_up)) + b_down."""
-    a = rnd(gelu_tanh(linear(h, w[p + "up"], w[p + "up.b"], dt, keep32=True)), dt)
+    a = rnd(gelu_tanh(linear(h, w[p + "up"], w[p + "up.b"], dt)), dt)
     return linear(a, w[p + "down"], w[p + "down.b"], dt)
 
 

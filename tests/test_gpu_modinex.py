@@ -1,0 +1,491 @@
+"""Modinex on the GPU against the plain implementation (``tests/plain/modinex_plain.py``): every mechanism alone,
+then whole models through the replay session and the engine: whole prompts, prefill + decoding, portions down to
+two tokens, mixed batches with pages and state slots used again, keys at the edges of chunks and pages, long
+decoding, greedy generation through the scheduler."""
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+from conftest import random_ids
+from modinex_cases import CASES, X, Y
+from plain import modinex_plain as M
+from tolerances import F32_REL
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTS = [torch.float32, torch.bfloat16]
+NAMES = {torch.float32: "float32", torch.bfloat16: "bfloat16"}
+
+
+def q(x, dt):
+    return x.to(dt).float()
+
+
+def close(got, want, dt, what, bf16=2.0 ** -7):
+    """float32: 2e-5 of the largest value (sum orders differ). bfloat16: a few roundings of the largest value."""
+    assert got.shape == want.shape and torch.isfinite(got).all(), f"{what}: shape or non-finite values"
+    scale = float(want.abs().max())
+    bound = (F32_REL if dt == torch.float32 else bf16) * max(scale, 1e-6)
+    err = float((got - want).abs().max())
+    assert err <= bound, f"{what}: max |diff| {err:.3e} > {bound:.3e} (largest value {scale:.3g})"
+
+
+# ----------------------------------------------------------------------------------------------- mechanisms alone
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("hidden,groups", [(96, 3), (96, 1), (200, 8), (1024, 2), (60, 5)])
+def test_norm_in_groups_around_a_sublayer(dt, hidden, groups):
+    from tokenmill_amd.parts import GroupRMSNorm, NormedInput, as_tensor
+    torch.manual_seed(hidden + groups)
+    T, eps = 7, 2e-5
+    pre, post = GroupRMSNorm(hidden, eps, groups, name=""), GroupRMSNorm(hidden, eps, groups, name="")
+    w1, w2 = q(torch.rand(hidden) + 0.5, dt), q(torch.randn(hidden), dt)
+    pre.load({"a": w1.to(dt).to(DEV)}, "a")
+    post.load({"b": w2.to(dt).to(DEV)}, "b")
+    resid, y = torch.randn(T, hidden) * 3, q(torch.randn(T, hidden) * 5, dt)
+    # the norm alone
+    r = resid.to(DEV)
+    got = pre.add_norm(r, None, dt)
+    close(got.float().cpu(), q(M.group_rms_norm(resid, w1, eps, groups), dt), dt, "norm alone", bf16=2.0 ** -8)
+    assert torch.equal(r.cpu(), resid)
+    # a pending result that passes its own norm: added, and the sum normed, in one call
+    x = NormedInput(pre, r, y.to(dt).to(DEV), dt, delta_norm=post)
+    got = as_tensor(x)
+    summed = resid + M.group_rms_norm(y, w2, eps, groups)
+    close(r.cpu(), summed, torch.float32, "residual after the result's norm")
+    close(got.float().cpu(), q(M.group_rms_norm(summed, w1, eps, groups), dt), dt, "norm of the sum", bf16=2.0 ** -8)
+    # the same for chosen rows only: the residual stays as it is
+    r2 = resid.to(DEV)
+    rows = torch.tensor([5, 0, 5, 2], dtype=torch.int32, device=DEV)
+    got = pre.add_norm(r2, y.to(dt).to(DEV), dt, rows=rows, delta_norm=post)
+    close(got.float().cpu(), q(M.group_rms_norm(summed, w1, eps, groups), dt)[rows.cpu().long()], dt, "chosen rows", bf16=2.0 ** -8)
+    assert torch.equal(r2.cpu(), resid)
+    # a result's norm of another shape than the next norm: two kernels, the same numbers
+    other = GroupRMSNorm(hidden, eps * 3, 1, name="")
+    other.load({"b": w2.to(dt).to(DEV)}, "b")
+    r3 = resid.to(DEV)
+    got = pre.add_norm(r3, y.to(dt).to(DEV), dt, delta_norm=other)
+    summed3 = resid + M.group_rms_norm(y, w2, eps * 3, 1)
+    close(r3.cpu(), summed3, torch.float32, "residual, another norm behind")
+    close(got.float().cpu(), q(M.group_rms_norm(summed3, w1, eps, groups), dt), dt, "norm, another norm behind", bf16=2.0 ** -8)
+    # the result's norm by itself
+    r4 = resid.to(DEV)
+    post.add_normed(r4, y.to(dt).to(DEV))
+    close(r4.cpu(), summed, torch.float32, "add_normed")
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_embedding_with_learned_positions_and_gelu(dt):
+    from tokenmill_amd.hip import ops
+    from tokenmill_amd.parts import LearnedPositions, TokenEmbedding
+    torch.manual_seed(1)
+    emb = TokenEmbedding(50, 72, name="embed", places=LearnedPositions(30, 72, name="pos"))
+    assert set(emb.tensor_specs("")) == {"embed", "pos"} and emb.by_position
+    e, p = q(torch.randn(50, 72), dt), q(torch.randn(30, 72), dt)
+    emb.load({"embed": e.to(dt).to(DEV), "pos": p.to(dt).to(DEV)}, "")
+    ids = torch.tensor([3, 49, 0, 3], dtype=torch.int32, device=DEV)
+    pos = torch.tensor([0, 29, 7, 8], dtype=torch.int32, device=DEV)
+    got = emb.forward(ids, pos)
+    assert got.dtype == torch.float32
+    assert torch.equal(got.cpu(), e[ids.cpu().long()] + p[pos.cpu().long()])       # one 32-bit sum of two exact values
+    for n in (5, 64, 1000):
+        z = q(torch.randn(n, 8) * 3, dt)
+        out = torch.empty_like(z.to(dt).to(DEV))
+        ops.gelu_tanh(z.to(dt).to(DEV), out)
+        close(out.float().cpu(), q(M.gelu_tanh(z), dt), dt, "gelu", bf16=2.0 ** -8)
+
+
+def _attention_fixture(dt, H, G, D, Dv, rot_dims, chunk, eps=1e-5, page=8, pages=64, max_pos=512, base=1e4, scale=0.3):
+    """A SigmoidAttention with random weights, its pools and manager, and its plain weights."""
+    from tokenmill_amd.cache import CacheManager
+    from tokenmill_amd.cache.pool import CachePools
+    from tokenmill_amd.engine.runner import ModelRunner
+    from tokenmill_amd.parts import RotaryEmbedding, SigmoidAttention
+    from test_gpu_parts import OneLayer
+    hidden = 64
+    rotary = RotaryEmbedding(D, base, max_pos, rotary_dim=rot_dims) if rot_dims else None
+    attn = SigmoidAttention(hidden, H, G, D, Dv, scale, rotary=rotary, qk_norm_eps=eps, chunk=chunk)
+    w = {}
+    for name, spec in attn.tensor_specs("a.").items():
+        w[name] = q((torch.rand(spec.shape) + 0.5) if spec.init == "ones" else torch.randn(spec.shape) * 0.3, dt)
+    attn.load({k: v.to(dt).to(DEV) for k, v in w.items()}, "a.")
+    attn.prepare(True)
+    pools = CachePools(OneLayer(attn), pages, page, 4, dt, DEV)
+    manager = CacheManager(pools.group_specs, pages, page, 4)
+
+    class Shell:
+        device = torch.device(DEV)
+
+        class head:
+            vocab = 10
+
+    runner = ModelRunner(Shell, pools, max_positions=max_pos)
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": Dv, "scale": scale}
+    if rot_dims:
+        m["rot"] = {"base": base, "dims": rot_dims}
+    if chunk:
+        m["mask"] = {"size": chunk}
+    return attn, w, m, pools, manager, runner, hidden
+
+
+def _run_cuts(attn, pools, manager, runner, x, dt, cuts):
+    from tokenmill_amd.engine.runner import StepEntry
+    rc = manager.allocate("r", 1)
+    outs, start = [], 0
+    for n in cuts:
+        manager.append(rc, start + n)
+        ctx, _ = runner.prepare([StepEntry(rc, start, [0] * n, [])])
+        outs.append(attn.forward(x[start:start + n].to(dt).to(DEV), ctx, pools.views[0]).float().cpu())
+        start += n
+        manager.release_behind_window(rc, start)
+    manager.free(rc)
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("H,G,D,Dv,rot,chunk", [(6, 2, 24, 16, 12, 24), (4, 4, 32, 40, 32, 50), (5, 1, 20, 68, 0, None),
+                                                 (2, 1, 128, 128, 64, 100), (3, 3, 6, 2, 2, 1)])
+def test_sigmoid_attention_whole_then_portions_then_tokens(dt, H, G, D, Dv, rot, chunk):
+    torch.manual_seed(7)
+    attn, w, m, pools, manager, runner, hidden = _attention_fixture(dt, H, G, D, Dv, rot, chunk)
+    L = 117
+    x = q(torch.randn(L, hidden), dt)
+    want = M.attention_mixer(x, w, "a.", m, 1e-5, dt)
+    for cuts in ([L], [40, 2, 7, 1, 1, 1, 30, 3, 32], [1] * 30 + [87]):
+        got = _run_cuts(attn, pools, manager, runner, x, dt, cuts)
+        close(got, want, dt, f"sigmoid attention {H, G, D, Dv, rot, chunk}, cuts {cuts[:4]}..")
+    manager.check_invariants()
+    assert manager.num_free_pages == manager.num_pages
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("single", [False, True])
+def test_keys_at_the_edges_of_chunks_and_pages_show(dt, single):
+    """Values are made so that every key shows in the output by itself: key j's value is 2^(j mod 20) in channel
+    j mod Dv of a one-hot, all scores are zero (the weights are sigmoid(pb) for every visible key), so the output
+    of a query names exactly the keys it summed: one too many or one too few at a chunk's start, a page's edge or
+    the query's own place changes a channel by a power of two."""
+    from tokenmill_amd.engine.runner import StepEntry
+    torch.manual_seed(8)
+    H, G, D, Dv, chunk, page = 2, 1, 8, 24, 21, 8
+    attn, w, m, pools, manager, runner, hidden = _attention_fixture(dt, H, G, D, Dv, 0, chunk, page=page)
+    L = 100
+    # q = 0 (zero matrix) makes every score zero; v is read from the input: W_v picks channels of x
+    dev = {k: v.clone() for k, v in w.items()}
+    dev["a.q"].zero_()
+    dev["a.v"].zero_()
+    dev["a.v"][:, :Dv] = torch.eye(Dv)
+    dev["a.o"].zero_()
+    dev["a.o"][:H * Dv, :] = 0
+    o = torch.zeros(hidden, H * Dv)
+    o[:Dv, :Dv] = torch.eye(Dv)                                            # head 0 shows in the first Dv channels of the result
+    o[Dv:2 * Dv, Dv:] = torch.eye(Dv)
+    dev["a.o"] = o
+    dev["a.pb"] = torch.tensor([0.0, 100.0])                               # weights 0.5 and 1
+    attn.load({k: v.to(dt).to(DEV) for k, v in dev.items()}, "a.")
+    x = torch.zeros(L, hidden)
+    for j in range(L):
+        x[j, j % Dv] = 2.0 ** (j % 7)
+    cuts = [1] * L if single else [19, 2, 1, 20, 22, 2, 34]
+    got = _run_cuts(attn, pools, manager, runner, x, dt, cuts)
+    for i in range(L):
+        want = torch.zeros(Dv)
+        for j in range(i // chunk * chunk, i + 1):
+            want[j % Dv] += 2.0 ** (j % 7)
+        assert torch.equal(got[i, :Dv], 0.5 * want), f"head 0, query {i}: {got[i, :Dv]} != {0.5 * want}"
+        assert torch.equal(got[i, Dv:2 * Dv], want), f"head 1, query {i}"
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_one_far_key_among_hundreds_stands_out(dt):
+    """No chunks: 300 keys; one early key is made to match the last queries (its k and their q share a large
+    component) while all other scores are strongly negative through the head bias, so the output is that key's value
+    or, if the key is lost, nothing."""
+    torch.manual_seed(9)
+    H, G, D, Dv = 2, 1, 16, 12
+    attn, w, m, pools, manager, runner, hidden = _attention_fixture(dt, H, G, D, Dv, 0, None, page=16, scale=1.0)
+    dev = {k: v.clone() for k, v in w.items()}
+    dev["a.pb"] = torch.tensor([-30.0, -30.0])
+    dev["a.q.norm"] = torch.ones(D)
+    dev["a.k.norm"] = torch.ones(D)
+    dev["a.q"] = torch.zeros(H * D, hidden)
+    dev["a.k"] = torch.zeros(G * D, hidden)
+    dev["a.q"][0, 0] = dev["a.q"][D, 0] = 1.0                              # channel 0 of x drives q[.., 0] of both heads
+    dev["a.k"][0, 1] = 1.0                                                 # channel 1 of x drives k[0]
+    attn.load({k: v.to(dt).to(DEV) for k, v in dev.items()}, "a.")
+    L, far = 300, 5
+    x = q(torch.randn(L, hidden) * 0.1, dt)
+    x[:, 0] = 0
+    x[:, 1] = 0
+    x[far, 1] = 8.0                                                        # after the norm: k = sqrt(D) e_0 for the far key only
+    x[-3:, 0] = 8.0                                                        # the last three queries look for it: score 16 * D^0 ...
+    want = M.attention_mixer(x, dev, "a.", m, 1e-5, dt)
+    assert float(want[-1].abs().max()) > 100 * float(want[100].abs().max())        # the far key is what the last rows are made of
+    for cuts in ([L], [290] + [1] * 10, [2] * 150):
+        close(_run_cuts(attn, pools, manager, runner, x, dt, cuts), want, dt, f"far key, cuts {cuts[:3]}")
+
+
+def _gla_fixture(dt, hidden, H, D, Dv, tau, rank, slots=4):
+    from tokenmill_amd.cache import CacheManager
+    from tokenmill_amd.cache.pool import CachePools
+    from tokenmill_amd.engine.runner import ModelRunner
+    from tokenmill_amd.parts import GatedLinearAttention
+    from test_gpu_parts import OneLayer
+    gla = GatedLinearAttention(hidden, H, D, Dv, tau, 1e-5, drawn_gate_rank=rank)
+    w = {}
+    for name, spec in gla.tensor_specs("g.").items():
+        shape = spec.drawn_shape()
+        w[name] = q((torch.rand(shape) + 0.5) if spec.init == "ones" else torch.randn(shape) * 0.4, dt)
+    gla.load({k: v.to(dt).to(DEV) for k, v in w.items()}, "g.")
+    pools = CachePools(OneLayer(gla), 8, 16, slots, dt, DEV)
+    manager = CacheManager(pools.group_specs, 8, 16, slots)
+
+    class Shell:
+        device = torch.device(DEV)
+
+        class head:
+            vocab = 10
+
+    return gla, w, pools, manager, ModelRunner(Shell, pools, max_positions=4096)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("H,D,Dv,tau,rank", [(2, 20, 24, 7.0, 5), (3, 36, 16, 3.0, 16), (1, 68, 12, 1.5, 1), (4, 8, 72, 20.0, 9),
+                                              (2, 128, 128, 16.0, 16), (1, 3, 1, 1.0, 2)])
+def test_gla_whole_then_portions_then_tokens_and_two_requests_side_by_side(dt, H, D, Dv, tau, rank):
+    from tokenmill_amd.engine.runner import StepEntry
+    torch.manual_seed(10)
+    hidden = 48
+    gla, w, pools, manager, runner = _gla_fixture(dt, hidden, H, D, Dv, tau, rank)
+    m = {"heads": H, "dim": D, "vdim": Dv, "tau": tau}
+    La, Lb = 83, 31
+    xa, xb = q(torch.randn(La, hidden), dt), q(torch.randn(Lb, hidden), dt)
+    want_a, Sa = M.gla_mixer(xa, w, "g.", m, 1e-5, dt, return_state=True)
+    want_b = M.gla_mixer(xb, w, "g.", m, 1e-5, dt)
+    for cuts in ([La], [30, 2, 1, 1, 1, 40, 8], [1] * La):
+        rc = manager.allocate("a", La)
+        pools.reset_state_slot(rc.state_slot)
+        outs, start = [], 0
+        for n in cuts:
+            ctx, _ = runner.prepare([StepEntry(rc, start, [0] * n, [])])
+            outs.append(gla.forward(xa[start:start + n].to(dt).to(DEV), ctx, pools.views[0]).float().cpu())
+            start += n
+        close(torch.cat(outs), want_a, dt, f"gla {H, D, Dv}, cuts {cuts[:3]}", bf16=2.0 ** -6)
+        close(pools.views[0].state[rc.state_slot].cpu(), Sa, dt, "gla state after the last token", bf16=2.0 ** -6)
+        manager.free(rc)
+    # two requests in one step, in slots that are not the first, one of them half done already
+    spare = manager.allocate("spare", 1)
+    ra, rb = manager.allocate("a", La), manager.allocate("b", Lb)
+    for r in (ra, rb):
+        pools.reset_state_slot(r.state_slot)
+    ctx, _ = runner.prepare([StepEntry(rb, 0, [0] * 10, [])])
+    first = gla.forward(xb[:10].to(dt).to(DEV), ctx, pools.views[0]).float().cpu()
+    ctx, _ = runner.prepare([StepEntry(rb, 10, [0] * (Lb - 10), []), StepEntry(ra, 0, [0] * La, [])])
+    both = gla.forward(torch.cat([xb[10:], xa]).to(dt).to(DEV), ctx, pools.views[0]).float().cpu()
+    close(torch.cat([first, both[:Lb - 10]]), want_b, dt, "gla, request b beside a", bf16=2.0 ** -6)
+    close(both[Lb - 10:], want_a, dt, "gla, request a beside b", bf16=2.0 ** -6)
+
+
+def test_gla_decays_and_a_state_that_fades_or_stays():
+    """Decays close to 1 keep a key for hundreds of tokens, small ones forget it at once: the recurrence kernel
+    against the plain loop with decays given directly."""
+    from tokenmill_amd.hip import ops
+    torch.manual_seed(11)
+    T, H, D, Dv = 400, 2, 12, 20
+    z = torch.randn(T, H * D) * 6
+    for tau in (1.0, 16.0):
+        got = ops.gla_decay(z.to(DEV).clone(), tau).cpu()
+        torch.testing.assert_close(got, torch.sigmoid(z.double()).pow(1 / tau).float(), rtol=2e-6, atol=1e-30)
+    decay = torch.rand(T, H, D)
+    decay[:, 0, :6] = 0.9995                                               # slow channels
+    decay[:, 1, 6:] = 1e-4                                                 # channels that forget
+    proj = torch.randn(T, 2 * H * D + H * Dv + 7)
+    qq, kk, vv = proj[:, 5:5 + H * D], proj[:, 5 + H * D:5 + 2 * H * D], proj[:, 5 + 2 * H * D:5 + 2 * H * D + H * Dv]
+    want, S = M.gla_recurrence(qq.reshape(T, H, D) * 0.5, kk.reshape(T, H, D), vv.reshape(T, H, Dv), decay.log())
+    state = torch.zeros(3, H, D, Dv, device=DEV)
+    o = torch.empty(T, H * Dv, device=DEV)
+    cu = torch.tensor([0, 150, T], dtype=torch.int32, device=DEV)
+    # the sequence as two portions of one request is not what cu means: two requests. So run it as one request in two calls.
+    for lo, hi in ((0, 150), (150, T)):
+        ops.gla_scan(proj[lo:hi].to(DEV), 5, 5 + H * D, 5 + 2 * H * D, decay[lo:hi].reshape(-1, H * D).to(DEV).contiguous(),
+                     o[lo:hi], state, torch.tensor([0, hi - lo], dtype=torch.int32, device=DEV),
+                     torch.tensor([2], dtype=torch.int32, device=DEV), 1, H, D, Dv, 0.5)
+    torch.testing.assert_close(o.cpu().view(T, H, Dv), want, rtol=2e-4, atol=2e-4)
+    torch.testing.assert_close(state[2].cpu(), S, rtol=2e-4, atol=2e-4)
+    assert float(state[:2].abs().max()) == 0.0                             # the other slots were not touched
+    del cu
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_dense_feed_forward_part(dt):
+    from tokenmill_amd.parts import DenseFeedForward
+    torch.manual_seed(12)
+    hidden, inter = 120, 200
+    ffn = DenseFeedForward(hidden, inter, suffixes=("", ".b"))
+    assert set(ffn.tensor_specs("m.")) == {"m.up", "m.up.b", "m.down", "m.down.b"}
+    w = {n: q(torch.randn(s.shape) * 0.2, dt) for n, s in ffn.tensor_specs("m.").items()}
+    ffn.load({k: v.to(dt).to(DEV) for k, v in w.items()}, "m.")
+    for T in (3, 90):
+        x = q(torch.randn(T, hidden), dt)
+        close(ffn.forward(x.to(dt).to(DEV)).float().cpu(), M.dense_ff(x, w, "m.", dt), dt, f"dense feed-forward, {T} rows")
+
+
+# ----------------------------------------------------------------------------------------------- whole models
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """name -> (folder, config, plain weights)"""
+    from tokenmill_amd.weights import write_random_model
+    out = {}
+    for name, (cfg, seed, std, norm_std) in CASES.items():
+        d = write_random_model(cfg, tmp_path_factory.mktemp(f"modinex{name}"), seed=seed, std=std, norm_std=norm_std)
+        out[name] = (d, *M.read_weights(d))
+    return out
+
+
+_plain_cache: dict = {}
+
+
+def plain_logits(models, name, ids, dt):
+    key = (name, tuple(ids), dt)
+    if key not in _plain_cache:
+        _, cfg, w = models[name]
+        _plain_cache[key] = M.logits(w, cfg, ids, dt)
+    return _plain_cache[key]
+
+
+def check_rows(models, name, got, reqs, dt, what):
+    """Every row against the plain row. float32: 5e-5 of the largest logit (the norm behind the recurrence divides a
+    first token's result by its own size, q.k times the value, and q.k can nearly cancel: the 32-bit rounding of that
+    dot product is then a larger share of it than of a sum that does not cancel). bfloat16: the engine may be as far
+    from the plain bfloat16 run as that run is from the plain float32 run (both differ from it by the same roundings,
+    falling differently), measured per request."""
+    assert got, "no rows"
+    for (rid, p), row in sorted(got.items()):
+        want = plain_logits(models, name, reqs[rid], dt)
+        if dt == torch.float32:
+            bound = 2.5 * F32_REL * float(want.abs().max())
+        else:
+            bound = 1.5 * float((want - plain_logits(models, name, reqs[rid], torch.float32)).abs().max())
+        err = float((row - want[p]).abs().max())
+        assert torch.isfinite(row).all() and err <= bound, f"{what}: request {rid} position {p}: {err:.3e} > {bound:.3e}"
+
+
+def make_requests(name, lengths, seed):
+    vocab = CASES[name][0]["vocab"]
+    return {f"r{i}": random_ids(n, vocab, seed * 100 + i) for i, n in enumerate(lengths)}
+
+
+def poison_freed_slots(session):
+    """A state slot that goes back is filled with NaN: a request that starts from anything but zero shows."""
+    slots, pools = session.manager.slots, session.pools
+    plain_release = slots.release
+
+    def release(slot):
+        for t in pools.states.values():
+            t[slot].fill_(math.nan)
+        return plain_release(slot)
+
+    slots.release = release
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", [("X", 16), ("Y", 8), ("X", 4)])
+def test_whole_decode_portions_mixed(models, name, page, dtype_name):
+    from tokenmill_amd.replay import ReplaySession
+    from test_gpu_replay import assert_all_given_back, mixed, poison_freed_pages, portions, prefill_then_decode, run_trace, whole
+    dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name]
+    s = ReplaySession(models[name][0], dtype_name, 4 * 128, page_size=page)
+    assert len(s.pools.states) == 2 and len(s.pools.groups) == 2
+    poison_freed_pages(s)
+    poison_freed_slots(s)
+    lengths = [1, 9, 26, 53, 120]
+    reqs = make_requests(name, lengths, 1)
+    got = run_trace(s, whole(reqs))
+    assert len(got) == sum(lengths)
+    check_rows(models, name, got, reqs, dt, "whole")
+    assert_all_given_back(s)
+    check_rows(models, name, run_trace(s, prefill_then_decode(reqs, tail=60)), reqs, dt, "prefill + decode")
+    assert_all_given_back(s)
+    steps = portions({k: v for k, v in reqs.items() if len(v) >= 2})
+    assert min(len(e["tokens"]) for st in steps for e in st["entries"]) == 2
+    check_rows(models, name, run_trace(s, steps), reqs, dt, "portions")
+    assert_all_given_back(s)
+    many = make_requests(name, [37, 64, 21, 90, 48, 33, 75, 18, 59, 44, 96, 27, 70, 52, 85, 40, 113, 66], 2)
+    steps = mixed(many, seed=5)
+    assert max(len(st["entries"]) for st in steps) == 4
+    got = run_trace(s, steps)
+    assert len(got) == sum(len(v) for v in many.values())
+    check_rows(models, name, got, many, dt, "mixed")
+    assert_all_given_back(s)
+    assert s.manager.slots.num_free == s.manager.slots.num_slots
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_long_decoding_over_chunks_with_their_pages_given_back(models, dtype_name):
+    """One token at a time from the third token on, to the model's last position: every chunk edge of both attention
+    layers and every page edge is passed by a decoded token; the pages of finished chunks go back on the way."""
+    from tokenmill_amd.replay import ReplaySession
+    from test_gpu_replay import assert_all_given_back, poison_freed_pages, run_trace
+    dt = {"float32": torch.float32, "bfloat16": torch.bfloat16}[dtype_name]
+    s = ReplaySession(models["X"][0], dtype_name, 256, page_size=8)
+    poison_freed_pages(s)
+    ids = random_ids(256, 211, 77)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": ids[:3], "want": [0, 1, 2]}], "end": []}]
+    steps += [{"step": p - 2, "entries": [{"id": "a", "tokens": [ids[p]], "want": [0]}], "end": ["a"] if p == 255 else []}
+              for p in range(3, 256)]
+    got, held = {}, []
+    for st in steps:
+        got.update(run_trace(s, [st]))
+        if "a" in s.manager.live:
+            held.append(sum(p != -1 for p in s.manager.live["a"].tables[0]))
+    check_rows(models, "X", got, {"a": ids}, dt, "long decoding")
+    assert max(held) <= 24 // 8 + 1, "the group with chunks of 24 never holds more than a chunk's pages and one"
+    assert_all_given_back(s)
+
+
+def test_greedy_generation_through_the_engine_and_its_graphs(models):
+    """The engine's own entry point: scheduler, chunked prefill, sampling, HIP graphs for the decode steps. Every token
+    is the plain implementation's first choice at its place (or a near-tie with it), and all modes agree."""
+    from tokenmill_amd import EngineConfig, LLMEngine, SamplingParams
+    d, cfg, w = models["X"]
+    prompts = [random_ids(n, 211, 500 + i) for i, n in enumerate([12, 3, 30, 7, 21, 16, 45, 25, 5, 18])]
+    params = [SamplingParams(max_tokens=8 + 5 * (i % 4), ignore_eos=True) for i in range(len(prompts))]
+    outs = {}
+    for mode in ("eager", "graphs", "chunked"):
+        eng = LLMEngine(EngineConfig(model=str(d), dtype="float32", block_size=8, num_blocks=48, max_model_len=96,
+                                     max_num_seqs=4, max_num_batched_tokens=32 if mode == "chunked" else 64, watermark=0.0,
+                                     hip_graphs=mode != "eager", enable_chunked_prefill=mode == "chunked"))
+        kinds = [type(p).__name__ for p in eng.runner.program.foreign_parts]
+        assert kinds.count("GatedLinearAttention") == 2 and kinds.count("SigmoidAttention") == 2
+        outs[mode] = eng.generate(prompts, params)
+        if mode == "graphs":
+            assert eng.runner.graphs.stateful_ok and eng.runner.graphs.replays > 10
+        assert eng.cache.num_free_pages == eng.cache.num_pages
+    tokens = {m: [list(o) for o in outs[m]] for m in outs}
+    assert tokens["eager"] == tokens["graphs"] == tokens["chunked"]
+    exempt = 0
+    for prompt, toks in zip(prompts, tokens["eager"]):
+        rows = M.logits(w, cfg, prompt + toks[:-1], torch.float32)[len(prompt) - 1:]
+        for row, tok in zip(rows, toks):
+            best = int(row.argmax())
+            if tok != best:
+                assert float(row[best] - row[tok]) <= 4 * F32_REL * float(row.abs().max()), "a token that is no near-tie"
+                exempt += 1
+    assert exempt <= 2
+
+
+def test_command_line_generates_with_a_random_modinex_model(tmp_path):
+    import json
+    import subprocess
+    import sys
+    from conftest import ROOT
+    (tmp_path / "config.json").write_text(json.dumps(Y))
+    r = subprocess.run([sys.executable, "-m", "tokenmill_amd.generate", "--random", str(tmp_path / "config.json"), "--prompt-ids",
+                        "5,9,33,2;7,7", "--max-tokens", "6", "--max-model-len", "64", "--ignore-eos"], capture_output=True, text=True, cwd=ROOT, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [json.loads(ln) for ln in r.stdout.splitlines() if ln.startswith("{")]
+    assert [len(ln["output_ids"]) for ln in lines] == [6, 6] and all(0 <= t < 150 for ln in lines for t in ln["output_ids"])

@@ -140,6 +140,13 @@ int tm_attn_sigmoid_paged(const void* q, int q_stride, void* out, int out_stride
                           const float* head_bias, int T, int H, int G, int D, int Dv, int page, float scale, int chunk,
                           int window, int dtype, hipStream_t stream);
 
+// The same attention for the prompt portions of a step on the matrix unit (attention_sigmoid_prefill.hip): bfloat16, the
+// step's tiles of up to 16 tokens as for tm_attn_prefill_mfma; tm_attn_sigmoid_prefill_takes says which sizes it runs.
+int tm_attn_sigmoid_prefill_takes(int D, int DV, int page, int q_stride);
+int tm_attn_sigmoid_prefill(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+                            const int* block_tables, int table_width, const int* tiles, int n_tiles, const float* head_bias,
+                            int H, int G, int D, int DV, int page, float scale, int chunk, int window, hipStream_t stream);
+
 // Gated linear attention (gla.hip): the decays from the gate projection, the recurrence over a step's rows request by
 // request with the state [slots, H, D, Dv] in 32-bit, and the per-head norm of the result times silu(gate).
 int tm_gla_decay(const float* z, float* a, float tau, long long n, hipStream_t stream);

@@ -1181,3 +1181,37 @@ def gla_out_gate(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, y: torch.
     _check(library().tm_gla_out_gate(_p(o), _p(gate), c_int(ldg), c_int(code(y.dtype)), _p(w), _p(y), c_int(T), c_int(H), c_int(Dv),
                                      c_float(eps), _stream()), "gla_out_gate")
     return y
+
+
+def attn_sigmoid_prefill_takes(dtype, D: int, Dv: int, page: int, q_stride: int) -> bool:
+    """Does the matrix-unit kernel for prompt portions run these sizes?"""
+    return dtype == torch.bfloat16 and bool(library().tm_attn_sigmoid_prefill_takes(c_int(D), c_int(Dv), c_int(page), c_int(q_stride)))
+
+
+def attn_sigmoid_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                         block_tables: torch.Tensor, tiles: torch.Tensor, head_bias: torch.Tensor | None, H: int, G: int,
+                         D: int, Dv: int, scale: float, chunk: int = 0, window: int = 0) -> torch.Tensor:
+    """``attn_sigmoid_paged`` for the rows of a step's prompt portions, given as tiles int32 [n, 4] = (request, first row,
+    tokens (1..16), position of the first token); bfloat16 on the matrix unit. Rows that belong to no tile are not written."""
+    _gpu(q, out, k_pool, v_pool, block_tables, tiles, head_bias)
+    T = q.shape[0]
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "attention(sigmoid, prefill): bfloat16 only")
+    _need(q.stride(1) == 1 and q.shape[1] >= H * D and out.is_contiguous() and tuple(out.shape) == (T, H * Dv),
+          f"attention(sigmoid, prefill): q [T, >={H * D}] unit inner stride, out contiguous [T, {H * Dv}]")
+    page = _check_pools_kv(k_pool, v_pool, G, D, Dv, q.dtype, "attention(sigmoid, prefill)")
+    q_stride = q.stride(0) if T > 1 else max(q.stride(0), H * D)
+    _need(H % G == 0 and attn_sigmoid_prefill_takes(q.dtype, D, Dv, page, q_stride) and q.data_ptr() % 16 == 0,
+          f"attention(sigmoid, prefill): sizes {D}/{Dv}, page {page}, row stride {q_stride} are not taken")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "attention(sigmoid, prefill): block_tables must be contiguous int32 [S, W]")
+    _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
+          "attention(sigmoid, prefill): tiles must be contiguous int32 [n, 4]")
+    if head_bias is not None:
+        _need(head_bias.dtype == torch.float32 and tuple(head_bias.shape) == (H,) and head_bias.is_contiguous(),
+              f"attention(sigmoid, prefill): head_bias is float32 [{H}]")
+    _need(chunk >= 0 and window >= 0, "attention(sigmoid, prefill): chunk and window must be >= 0")
+    _check(library().tm_attn_sigmoid_prefill(_p(q), c_int(q_stride), _p(out), c_int(H * Dv), _p(k_pool), _p(v_pool),
+                                             _p(block_tables), c_int(block_tables.shape[1]), _p(tiles), c_int(tiles.shape[0]),
+                                             _p(head_bias), c_int(H), c_int(G), c_int(D), c_int(Dv), c_int(page), c_float(scale),
+                                             c_int(chunk), c_int(window), _stream()), "attn_sigmoid_prefill")
+    return out

@@ -121,7 +121,25 @@ class SigmoidAttention(Mixer):
                                    cache.k if write else None, cache.v if write else None)
         out = torch.empty((T, H * Dv), dtype=x.dtype, device=x.device)
         with profiling.label("attention", lambda: self.cost("attention", step, T)):
-            ops.attn_sigmoid_paged(qkv, out, cache.k, cache.v, group.block_tables, step.seq_of_token, step.positions,
-                                   self.head_bias, H, G, D, Dv, self.scale, self.chunk or 0, self.window or 0)
+            self._attend(qkv, out, step, cache, group)
         with profiling.label("o_proj", lambda: self.o.cost(T)):
             return self.o.forward(out)
+
+    def _attend(self, qkv, out, step: StepContext, cache: KVCacheView, group) -> None:
+        """Prompt portions on the matrix unit where its kernel takes the sizes, single tokens (the step's last
+        ``num_decode`` rows) and everything else through the kernel that takes a token and a head a wavefront."""
+        H, G, D, Dv = self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim
+        T = qkv.shape[0]
+        tiles = step.prefill_tiles
+        first_single = T - step.num_decode
+        if (tiles is not None and tiles.shape[0] and first_single > 0 and qkv.data_ptr() % 16 == 0
+                and ops.attn_sigmoid_prefill_takes(qkv.dtype, D, Dv, cache.k.shape[1], qkv.stride(0))):
+            ops.attn_sigmoid_prefill(qkv, out, cache.k, cache.v, group.block_tables, tiles, self.head_bias, H, G, D, Dv,
+                                     self.scale, self.chunk or 0, self.window or 0)
+            if step.num_decode == 0:
+                return
+            rows = slice(first_single, T)
+        else:
+            rows = slice(0, T)
+        ops.attn_sigmoid_paged(qkv[rows], out[rows], cache.k, cache.v, group.block_tables, step.seq_of_token[rows],
+                               step.positions[rows], self.head_bias, H, G, D, Dv, self.scale, self.chunk or 0, self.window or 0)
