@@ -3,7 +3,7 @@ weights, synthetic token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
                     [--config CONFIG.json|NAME]      another shape of the architecture (7b, 32b, a file)
-                    [--part all|decode|prefill|offline|mixed7b|preempt32b]
+                    [--part all|decode|prefill|offline|mixed7b|preempt32b|modinex]
                     [--part decode --contexts 8192,32768 --batches 8,64]     decode steps over long contexts
 
 A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
@@ -19,6 +19,10 @@ of their operations has to move and do), not from formulas of one architecture.
                         (portions of prompts beside decoding requests, budget 2,048), up to 64 at a time
     --part preempt32b   the 32B shape, context 8,192: 64 prompts of 2,048 ids on 8,192 pages of 16, so
                         that growth during decoding evicts requests; reports evictions and tok/s
+    --part modinex      the Modinex design at two sizes that resemble a real model's layers (shipped shapes modinex-1k,
+                        modinex-2k), each beside the Qwen2 model of equal width, depth, heads and feed-forward
+                        parameters (qwen2-like-1k, qwen2-like-2k): prefill and decode rates, and per operation its
+                        GPU time and the share of its floor it reaches
 """
 from __future__ import annotations
 
@@ -38,6 +42,25 @@ PROMPT_LEN = 2048
 BLOCK_SIZE = 16
 HISTOGRAM_STEPS = 128            # the step-time histogram is taken over at least this many decode steps
 PROFILED_STEPS = 8               # decode steps run under the kernel trace
+
+
+def _linears(model):
+    """Every Linear part of a model (for a count of its matrix parameters)."""
+    from tokenmill_amd.parts import Linear
+    seen, stack, out = set(), [model], []
+    while stack:
+        obj = stack.pop()
+        if id(obj) in seen:
+            continue
+        seen.add(id(obj))
+        if isinstance(obj, Linear):
+            out.append(obj)
+            continue
+        if isinstance(obj, (list, tuple)):
+            stack.extend(obj)
+        elif hasattr(obj, "__dict__") and type(obj).__module__.startswith("tokenmill_amd"):
+            stack.extend(vars(obj).values())
+    return out
 
 
 def percentile(xs: list[float], p: float) -> float:
@@ -64,7 +87,7 @@ def main() -> int:
                     help="captured shapes also try every algorithm the library holds, not only its heuristic's candidates")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
     ap.add_argument("--skip-kernels", action="store_true", help="no per-operation kernel trace")
-    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b"],
+    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b", "modinex"],
                     help="all: the headline line. decode / prefill: only that (for profiling one of them). offline: "
                          "--requests prompts of --offline-prompt tokens submitted at once. mixed7b / preempt32b: see above")
     ap.add_argument("--requests", type=int, default=None, help="requests of the offline, mixed7b and preempt32b parts")
@@ -105,15 +128,15 @@ def main() -> int:
     shape, shape_name = read_shape(HEADLINE_SHAPE), "Qwen2.5-0.5B shape"
     if args.config:
         shape, shape_name = read_shape(args.config), Path(args.config).stem
-    layers_full = shape["num_hidden_layers"]
+    layers_full = shape.get("num_hidden_layers", len(shape.get("layers", [])))
     if args.layers:
         shape["num_hidden_layers"] = args.layers
     # the position tables reach the longest context any engine of this run allows (each engine has its own limit)
     most_positions = max([max_model_len] + sweep + ([] if args.skip_points or args.part != "all" else list(LONG_POINTS)))
     most_positions = min(most_positions, shape.get("max_position_embeddings", most_positions))
-    model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
+    model = None if args.part == "modinex" else load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
     gen = torch.Generator().manual_seed(0)
-    vocab = shape["vocab_size"]
+    vocab = model.head.vocab if model is not None else None
 
     def prompts(n, length=None):
         return [torch.randint(0, vocab, (length or prompt_len,), generator=gen).tolist() for _ in range(n)]
@@ -330,6 +353,32 @@ def main() -> int:
                 "config": {**sizes(), "requests": n, "prompt": prompt_len, "gen": gen_tokens, "max_num_seqs": n,
                            "token_budget": 2048, "max_model_len": max_model_len, "block_size": BLOCK_SIZE, "pages": pages}}
 
+    if args.part == "modinex":
+        # the new design beside the closest existing model at equal size: the functions above measure whatever
+        # `model` is, so each shape is loaded in turn
+        rows = {}
+        for size in ("1k", "2k"):
+            for name in (f"modinex-{size}", f"qwen2-like-{size}"):
+                shape, shape_name = read_shape(name), name
+                model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
+                vocab = model.head.vocab
+                pre = time_prefill(detail=True)
+                dec = time_decode(args.batch, max(16, args.steps // 4), max(4, args.warmup // 2), detail=True)
+                params = sum(t.numel() for t in (getattr(lin, "weight", None) for lin in _linears(model)) if t is not None)
+                rows[name] = {"matrix_params": params,
+                              "prefill_tok_s": round(prompt_len / pre["s"], 1), "prefill_ms": round(pre["s"] * 1e3, 3),
+                              "prefill_mfma_frac": round(pre["flops"] / pre["s"] / profiling.PEAK_FLOPS_S[args.dtype], 4),
+                              "prefill_kernel_ms": pre.get("kernel_ms"), "prefill_kernels": pre.get("kernels"),
+                              "decode_tok_s": round(args.batch / dec["step_s"], 1), "decode_ms_per_step": round(dec["step_s"] * 1e3, 4),
+                              "decode_hbm_frac": round(dec["bytes"] / dec["step_s"] / profiling.PEAK_HBM_BYTES_S, 4),
+                              "decode_kernel_ms": dec.get("kernel_ms"), "decode_kernels": dec.get("kernels")}
+                print(f"{name}: {json.dumps(rows[name])}", file=sys.stderr, flush=True)
+                del model
+                model = None
+                torch.cuda.empty_cache()
+        print(json.dumps({"metric": f"Modinex beside Qwen2 at equal size: prefill of {prompt_len} tokens, decode at batch {args.batch}",
+                          "dtype": args.dtype, "prompt": prompt_len, "batch": args.batch, "rows": rows}))
+        return 0
     if args.part == "offline":
         print(json.dumps(time_offline()))
         return 0

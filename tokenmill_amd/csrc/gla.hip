@@ -9,8 +9,8 @@
 //   gla_scan      the recurrence; reads q, k, v from the rows of the stacked projection, writes o in 32-bit
 //   gla_out_gate  y = w * o / rms(o) (per head, over Dv) * silu(g), rounded once to the model's type
 // Everything that enters the recurrence is 32-bit. The columns of S are independent of each other, so the scan is
-// dealt over (request, head, 64 columns) blocks of four wavefronts; a lane keeps a quarter of a column's D rows in
-// registers, and a column's four partial dot products are added in a fixed order. A token's result depends on its request's state
+// dealt over (request, head, 16 columns) wavefronts; a lane keeps a quarter of a column's D rows in registers, and a
+// column's four partial dot products are added in a fixed order. A token's result depends on its request's state
 // and tokens only, never on the step's other rows or on how the prompt was cut.
 #include "common.h"
 #include "api.h"
@@ -34,95 +34,45 @@ extern "C" int tm_gla_decay(const float* z, float* a, float tau, long long n, hi
 
 #define GLA_PARTS 4                         // lanes that share a column's rows
 #define GLA_COLS (TM_WAVE / GLA_PARTS)      // columns of a wavefront
-#define GLA_WAVES 4                         // wavefronts of a block
-#define GLA_BLOCK_COLS (GLA_COLS * GLA_WAVES)
-#define GLA_THREADS (TM_WAVE * GLA_WAVES)
-#define GLA_MAX_PREFETCH 28                 // elements a thread holds of the next batch of tokens
 
-// grid (ceil(Dv / GLA_BLOCK_COLS), H, S); a block is four wavefronts of 16 columns each. lane = column * GLA_PARTS +
-// part; part p keeps rows p * R .. p * R + R - 1 of its column, R = ceil(D / GLA_PARTS) <= RMAX. The block stages
-// q (scaled), k, the decays and its columns of v of TB tokens at a time in LDS, as 32-bit floats: the next batch is
-// asked for before the current one is worked on and stored behind it, one barrier a batch.
+// grid (ceil(Dv / GLA_COLS), H, S); a block is one wavefront. lane = column * GLA_PARTS + part; part p keeps rows
+// p * R .. p * R + R - 1 of its column, R = ceil(D / GLA_PARTS) <= RMAX.
 template <typename T, int RMAX>
-__global__ __launch_bounds__(GLA_THREADS) void gla_scan_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off,
-                                                              int v_off, const float* __restrict__ decay,
-                                                              float* __restrict__ o, float* __restrict__ state,
-                                                              const int* __restrict__ cu_q_lens,
-                                                              const int* __restrict__ state_slots, int H, int D, int Dv,
-                                                              float q_scale, int TB) {
-    extern __shared__ float lds[];
-    const int W = 3 * D + GLA_BLOCK_COLS;             // floats of a staged token: q | k | decay | v columns
-    const int tid = threadIdx.x, lane = tid % TM_WAVE, wave = tid / TM_WAVE, part = lane % GLA_PARTS;
-    const int col0 = blockIdx.x * GLA_BLOCK_COLS;
-    const int cb = wave * GLA_COLS + lane / GLA_PARTS;      // column within the block
-    const int e = col0 + cb;
+__global__ __launch_bounds__(TM_WAVE) void gla_scan_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
+                                                          const float* __restrict__ decay, float* __restrict__ o,
+                                                          float* __restrict__ state, const int* __restrict__ cu_q_lens,
+                                                          const int* __restrict__ state_slots, int H, int D, int Dv,
+                                                          float q_scale) {
+    const int lane = threadIdx.x, part = lane % GLA_PARTS;
+    const int e = blockIdx.x * GLA_COLS + lane / GLA_PARTS;
     const int h = blockIdx.y, s = blockIdx.z;
     const int R = (D + GLA_PARTS - 1) / GLA_PARTS;
     const int d0 = part * R;
     const bool col = e < Dv;
     const int t0 = cu_q_lens[s], t1 = cu_q_lens[s + 1];
-    if (t1 <= t0) return;                                  // the whole block
+    if (t1 <= t0) return;
     float* st = state + (((size_t)state_slots[s] * H + h) * D) * Dv + (col ? e : 0);
     float S[RMAX];
 #pragma unroll
     for (int i = 0; i < RMAX; ++i) S[i] = (col && i < R && d0 + i < D) ? st[(size_t)(d0 + i) * Dv] : 0.f;
-
-    const int per_batch = TB * W;
-    float pf[GLA_MAX_PREFETCH];
-    auto fetch = [&](int tb) {                             // batch starting at token tb -> registers
+    for (int t = t0; t < t1; ++t) {
+        const T* row = proj + (size_t)t * ld;
+        const T* qr = row + q_off + h * D + d0;
+        const T* kr = row + k_off + h * D + d0;
+        const float* ar = decay + ((size_t)t * H + h) * D + d0;
+        const float v = col ? Elem<T>::load(row + v_off + h * Dv + e) : 0.f;
+        float acc = 0.f;
 #pragma unroll
-        for (int i = 0; i < GLA_MAX_PREFETCH; ++i) {
-            const int idx = tid + i * GLA_THREADS;
-            float v = 0.f;
-            if (idx < per_batch) {
-                const int j = idx / W, c = idx - j * W;
-                const int t = tb + j;
-                if (t < t1) {
-                    const T* row = proj + (size_t)t * ld;
-                    if (c < D) v = Elem<T>::load(row + q_off + h * D + c) * q_scale;
-                    else if (c < 2 * D) v = Elem<T>::load(row + k_off + h * D + (c - D));
-                    else if (c < 3 * D) v = decay[((size_t)t * H + h) * D + (c - 2 * D)];
-                    else if (col0 + (c - 3 * D) < Dv) v = Elem<T>::load(row + v_off + h * Dv + col0 + (c - 3 * D));
-                }
+        for (int i = 0; i < RMAX; ++i) {
+            if (i < R && d0 + i < D) {
+                const float kv = Elem<T>::load(kr + i) * v;
+                S[i] = ar[i] * S[i] + kv;
+                acc += S[i] * (Elem<T>::load(qr + i) * q_scale);
             }
-            pf[i] = v;
         }
-    };
-    auto stash = [&](float* buf) {
-#pragma unroll
-        for (int i = 0; i < GLA_MAX_PREFETCH; ++i) {
-            const int idx = tid + i * GLA_THREADS;
-            if (idx < per_batch) buf[idx] = pf[i];
-        }
-    };
-    fetch(t0);
-    stash(lds);
-    __syncthreads();
-    int which = 0;
-    for (int tb = t0; tb < t1; tb += TB) {
-        const float* buf = lds + which * per_batch;
-        const bool more = tb + TB < t1;
-        if (more) fetch(tb + TB);
-        const int n = min(TB, t1 - tb);
-        for (int j = 0; j < n; ++j) {
-            const float* row = buf + j * W;
-            const float v = row[3 * D + cb];
-            float acc = 0.f;
-#pragma unroll
-            for (int i = 0; i < RMAX; ++i) {
-                if (i < R && d0 + i < D) {
-                    const float kv = row[D + d0 + i] * v;
-                    S[i] = row[2 * D + d0 + i] * S[i] + kv;
-                    acc += S[i] * row[d0 + i];
-                }
-            }
-            acc += __shfl_xor(acc, 1, TM_WAVE);
-            acc += __shfl_xor(acc, 2, TM_WAVE);
-            if (col && part == 0) o[((size_t)(tb + j) * H + h) * Dv + e] = acc;
-        }
-        if (more) stash(lds + (which ^ 1) * per_batch);
-        __syncthreads();
-        which ^= 1;
+        acc += __shfl_xor(acc, 1, TM_WAVE);
+        acc += __shfl_xor(acc, 2, TM_WAVE);
+        if (col && part == 0) o[((size_t)t * H + h) * Dv + e] = acc;
     }
 #pragma unroll
     for (int i = 0; i < RMAX; ++i)
@@ -132,21 +82,17 @@ __global__ __launch_bounds__(GLA_THREADS) void gla_scan_kernel(const T* __restri
 template <typename T>
 static int launch_gla_scan(const void* proj, int ld, int q_off, int k_off, int v_off, const float* decay, float* o, float* state,
                            const int* cu, const int* slots, int S, int H, int D, int Dv, float q_scale, hipStream_t stream) {
-    const dim3 grid((Dv + GLA_BLOCK_COLS - 1) / GLA_BLOCK_COLS, H, S);
+    const dim3 grid((Dv + GLA_COLS - 1) / GLA_COLS, H, S);
     const int R = (D + GLA_PARTS - 1) / GLA_PARTS;
-    const int W = 3 * D + GLA_BLOCK_COLS;
-    int TB = 16;                                           // tokens a batch: what a thread's prefetch registers hold
-    while (TB > 1 && TB * W > GLA_MAX_PREFETCH * GLA_THREADS) TB /= 2;
-    const size_t lds = 2 * (size_t)TB * W * sizeof(float);
     if (R <= 16)
-        gla_scan_kernel<T, 16><<<grid, GLA_THREADS, lds, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu,
-                                                                  slots, H, D, Dv, q_scale, TB);
+        gla_scan_kernel<T, 16><<<grid, TM_WAVE, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu, slots, H,
+                                                            D, Dv, q_scale);
     else if (R <= 32)
-        gla_scan_kernel<T, 32><<<grid, GLA_THREADS, lds, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu,
-                                                                  slots, H, D, Dv, q_scale, TB);
+        gla_scan_kernel<T, 32><<<grid, TM_WAVE, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu, slots, H,
+                                                            D, Dv, q_scale);
     else
-        gla_scan_kernel<T, 64><<<grid, GLA_THREADS, lds, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu,
-                                                                  slots, H, D, Dv, q_scale, TB);
+        gla_scan_kernel<T, 64><<<grid, TM_WAVE, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu, slots, H,
+                                                            D, Dv, q_scale);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
