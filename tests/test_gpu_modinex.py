@@ -368,7 +368,7 @@ def plain_logits(models, name, ids, dt):
 def check_rows(models, name, got, reqs, dt, what):
     """Every row against the plain row. float32: 5e-5 of the largest logit (the norm behind the recurrence divides a
     first token's result by its own size, q.k times the value, and q.k can nearly cancel: the 32-bit rounding of that
-    dot product is then a larger share of it than of a sum that does not cancel). bfloat16: the engine may be as far
+    dot product is then a larger share of it than of a sum that does not cancel). bfloat16: the engine may be twice as far
     from the plain bfloat16 run as that run is from the plain float32 run (both differ from it by the same roundings,
     falling differently), measured per request."""
     assert got, "no rows"
@@ -377,7 +377,8 @@ def check_rows(models, name, got, reqs, dt, what):
         if dt == torch.float32:
             bound = 2.5 * F32_REL * float(want.abs().max())
         else:
-            bound = 1.5 * float((want - plain_logits(models, name, reqs[rid], torch.float32)).abs().max())
+            bound = max(2.0 * float((want - plain_logits(models, name, reqs[rid], torch.float32)).abs().max()),
+                        2.0 ** -7 * float(want.abs().max()))
         err = float((row - want[p]).abs().max())
         assert torch.isfinite(row).all() and err <= bound, f"{what}: request {rid} position {p}: {err:.3e} > {bound:.3e}"
 

@@ -50,6 +50,16 @@ __device__ __forceinline__ void sg_load_block(SgBlock<DP, DVP>& blk, int kb, int
                                               int page_shift, int r, int g) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
+        // A tile no query of the wavefront can see (wholly before the first visible key, or beyond the newest) is not
+        // loaded: its place in the table may name no page, and what another tile's slots hold beyond the newest key
+        // can be anything. Its keys and values are zeros; its weights are masked by position like any other's.
+        if (2 * kb + t < first_tile || 2 * kb + t > last_tile) {
+#pragma unroll
+            for (int c = 0; c < DP / 32; ++c) blk.k[t][c].u = u32x4_t{0, 0, 0, 0};
+#pragma unroll
+            for (int dt = 0; dt < DVP / 16; ++dt) blk.v[dt][t] = u32x2_t{0, 0};
+            continue;
+        }
         int pg, in_page;
         sg_tile_place(2 * kb + t, first_tile, last_tile, table, page_shift, pg, in_page);
         pg = __builtin_amdgcn_readfirstlane(pg);
