@@ -297,6 +297,45 @@ def test_gla_whole_then_portions_then_tokens_and_two_requests_side_by_side(dt, H
     close(both[Lb - 10:], want_a, dt, "gla, request a beside b", bf16=2.0 ** -6)
 
 
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("H,D,Dv,tau,rank", [(2, 20, 24, 7.0, 8), (2, 128, 128, 16.0, 16), (3, 36, 16, 2.0, 16)])
+def test_gla_long_portions_run_in_segments(dt, H, D, Dv, tau, rank):
+    """Portions of 128 rows and more are scanned in segments of 64 (from zero states, a chain over the segments, and
+    again from the true start states): the same results up to rounding, the same state behind them, whole, cut at
+    places that are no multiples of 64, and beside a request that is decoding."""
+    from tokenmill_amd.engine.runner import StepEntry
+    torch.manual_seed(13)
+    hidden = 48
+    gla, w, pools, manager, runner = _gla_fixture(dt, hidden, H, D, Dv, tau, rank)
+    assert gla.SEGMENT == 64
+    m = {"heads": H, "dim": D, "vdim": Dv, "tau": tau}
+    La, Lb = 333, 40
+    xa, xb = q(torch.randn(La, hidden), dt), q(torch.randn(Lb, hidden), dt)
+    want_a, Sa = M.gla_mixer(xa, w, "g.", m, 1e-5, dt, return_state=True)
+    want_b, Sb = M.gla_mixer(xb, w, "g.", m, 1e-5, dt, return_state=True)
+    for cuts in ([La], [150, 3, 129, 51], [128, 205]):
+        ra, rb = manager.allocate("a", 1), manager.allocate("b", 1)
+        for r in (ra, rb):
+            pools.reset_state_slot(r.state_slot)
+        ctx, _ = runner.prepare([StepEntry(rb, 0, [0] * (Lb - len(cuts)), [])])
+        outs_b = [gla.forward(xb[:Lb - len(cuts)].to(dt).to(DEV), ctx, pools.views[0]).float().cpu()]
+        outs_a, start = [], 0
+        for i, n in enumerate(cuts):                      # request b decodes one token beside every portion of a
+            pb_ = Lb - len(cuts) + i
+            ctx, _ = runner.prepare([StepEntry(rb, pb_, [0], []), StepEntry(ra, start, [0] * n, [])])
+            assert ctx.q_lens == [n, 1]                   # the portion stands first in the step
+            both = gla.forward(torch.cat([xa[start:start + n], xb[pb_:pb_ + 1]]).to(dt).to(DEV), ctx, pools.views[0]).float().cpu()
+            outs_a.append(both[:n])
+            outs_b.append(both[n:])
+            start += n
+        close(torch.cat(outs_a), want_a, dt, f"gla in segments {H, D, Dv}, cuts {cuts}", bf16=2.0 ** -6)
+        close(torch.cat(outs_b), want_b, dt, f"gla beside segments {H, D, Dv}, cuts {cuts}", bf16=2.0 ** -6)
+        close(pools.views[0].state[ra.state_slot].cpu(), Sa, dt, "state behind the segments", bf16=2.0 ** -6)
+        close(pools.views[0].state[rb.state_slot].cpu(), Sb, dt, "state of the request beside them", bf16=2.0 ** -6)
+        manager.free(ra)
+        manager.free(rb)
+
+
 def test_gla_decays_and_a_state_that_fades_or_stays():
     """Decays close to 1 keep a key for hundreds of tokens, small ones forget it at once: the recurrence kernel
     against the plain loop with decays given directly."""

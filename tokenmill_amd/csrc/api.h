@@ -155,6 +155,15 @@ int tm_gla_scan(const void* proj, int ld, int q_off, int k_off, int v_off, int d
                 hipStream_t stream);
 int tm_gla_out_gate(const float* o, const void* gate, int ldg, int dtype, const float* w, void* y, int T, int H, int Dv,
                     float eps, hipStream_t stream);
+// The decays straight from the narrow projection x [T, K] (rows ldx apart), W [N, K], bias [N] of the model's type:
+// a = sigmoid(x W^T + b)^(1/tau), 32-bit. And a long portion in segments (see gla.hip): the product of each segment's
+// decays, and the chain over a request's segments that turns the segments' local states into their true start states
+// and the request's new state.
+int tm_gla_gate_decay(const void* x, int ldx, const void* W, const void* bias, int dtype, float* a, int T, int N, int K,
+                      float tau, hipStream_t stream);
+int tm_gla_segment_decay(const float* decay, const int* cu_seg, float* P, int n_seg, int HD, hipStream_t stream);
+int tm_gla_combine(float* state, const int* state_slots, const int* first_seg, const float* P, const float* local,
+                   float* start, int S, int HD, int Dv, hipStream_t stream);
 
 int tm_argmax_work_chunks(int V);
 int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);

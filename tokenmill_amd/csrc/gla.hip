@@ -145,3 +145,98 @@ extern "C" int tm_gla_out_gate(const float* o, const void* gate, int ldg, int dt
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
+
+// ------------------------------------------------------------------------------------------------------------------
+// The decays straight from the narrow projection: a[t, n] = sigmoid(z)^(1/tau), z = sum_k x[t, k] W[n, k] + b[n], with
+// the sum and everything behind it in 32-bit. K is the gate's width (a handful of channels), so a thread per output
+// walks it in ascending k; the row of x is the same for all threads of a block.
+// ------------------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void gla_gate_decay_kernel(const T* __restrict__ x, int ldx, const T* __restrict__ W,
+                                                            const T* __restrict__ bias, float* __restrict__ a, int N, int K,
+                                                            float inv_tau) {
+    const int n = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+    if (n >= N) return;
+    const T* xr = x + (size_t)t * ldx;
+    const T* wr = W + (size_t)n * K;
+    float z = bias ? Elem<T>::load(bias + n) : 0.f;
+    for (int k = 0; k < K; ++k) z += Elem<T>::load(xr + k) * Elem<T>::load(wr + k);
+    const float ls = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+    a[(size_t)t * N + n] = expf(ls * inv_tau);
+}
+
+extern "C" int tm_gla_gate_decay(const void* x, int ldx, const void* W, const void* bias, int dtype, float* a, int T, int N,
+                                 int K, float tau, hipStream_t stream) {
+    if (T <= 0 || N <= 0) return TM_OK;
+    if (!x || !W || !a || K <= 0 || ldx < K || !(tau > 0.f) || T > 65535 * 32) return TM_ERR_ARG;
+    for (int t0 = 0; t0 < T; t0 += 65535) {
+        const int rows = T - t0 < 65535 ? T - t0 : 65535;
+        const dim3 grid((N + 255) / 256, rows);
+        if (dtype == TM_F32)
+            gla_gate_decay_kernel<float><<<grid, 256, 0, stream>>>((const float*)x + (size_t)t0 * ldx, ldx, (const float*)W,
+                                                                  (const float*)bias, a + (size_t)t0 * N, N, K, 1.0f / tau);
+        else if (dtype == TM_BF16)
+            gla_gate_decay_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x + (size_t)t0 * ldx, ldx, (const bf16_t*)W,
+                                                                   (const bf16_t*)bias, a + (size_t)t0 * N, N, K, 1.0f / tau);
+        else
+            return TM_ERR_ARG;
+        TM_CHECK_LAUNCH();
+    }
+    return TM_OK;
+}
+
+// ------------------------------------------------------------------------------------------------------------------
+// A long portion in segments. The recurrence is linear in the state, so a segment's rows can be worked on before the
+// state at its start is known: with the rows of a request cut into segments c = 0, 1, ...
+//   L_c = the state the segment's own rows build from zero          (tm_gla_scan over the segments, from zero states)
+//   P_c = the product of the segment's decays, per key channel      (gla_segment_decay)
+//   B_0 = the request's state, B_(c+1) = diag(P_c) B_c + L_c        (gla_combine; the last one is the request's new state)
+// and then every segment is scanned again from its true start B_c, all segments at once (tm_gla_scan once more).
+// The chain over tokens becomes a chain over segments plus two scans that fill the chip.
+// ------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gla_segment_decay_kernel(const float* __restrict__ decay, const int* __restrict__ cu_seg,
+                                                               float* __restrict__ P, int HD) {
+    const int j = blockIdx.x * 256 + threadIdx.x, c = blockIdx.y;
+    if (j >= HD) return;
+    float p = 1.f;
+    for (int t = cu_seg[c]; t < cu_seg[c + 1]; ++t) p *= decay[(size_t)t * HD + j];
+    P[(size_t)c * HD + j] = p;
+}
+
+// grid (ceil(H * D * Dv / 256), S): element (h, d, e) of request s walks the request's segments first_seg[s] ..
+// first_seg[s + 1] - 1 in order. local [n_seg, H, D, Dv] holds L_c; start receives B_c.
+__global__ __launch_bounds__(256) void gla_combine_kernel(float* __restrict__ state, const int* __restrict__ state_slots,
+                                                         const int* __restrict__ first_seg, const float* __restrict__ P,
+                                                         const float* __restrict__ local, float* __restrict__ start, int HD,
+                                                         int Dv) {
+    const size_t per = (size_t)HD * Dv;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= per) return;
+    const int s = blockIdx.y;
+    const size_t hd = idx / Dv;
+    float* st = state + (size_t)state_slots[s] * per + idx;
+    float S = *st;
+    for (int c = first_seg[s]; c < first_seg[s + 1]; ++c) {
+        start[(size_t)c * per + idx] = S;
+        S = P[(size_t)c * HD + hd] * S + local[(size_t)c * per + idx];
+    }
+    *st = S;
+}
+
+extern "C" int tm_gla_segment_decay(const float* decay, const int* cu_seg, float* P, int n_seg, int HD, hipStream_t stream) {
+    if (n_seg <= 0) return TM_OK;
+    if (!decay || !cu_seg || !P || HD <= 0 || n_seg > 65535) return TM_ERR_ARG;
+    gla_segment_decay_kernel<<<dim3((HD + 255) / 256, n_seg), 256, 0, stream>>>(decay, cu_seg, P, HD);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+extern "C" int tm_gla_combine(float* state, const int* state_slots, const int* first_seg, const float* P, const float* local,
+                              float* start, int S, int HD, int Dv, hipStream_t stream) {
+    if (S <= 0) return TM_OK;
+    if (!state || !state_slots || !first_seg || !P || !local || !start || HD <= 0 || Dv <= 0 || S > 65535) return TM_ERR_ARG;
+    const size_t per = (size_t)HD * Dv;
+    gla_combine_kernel<<<dim3((unsigned)((per + 255) / 256), S), 256, 0, stream>>>(state, state_slots, first_seg, P, local, start, HD, Dv);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}

@@ -1215,3 +1215,50 @@ def attn_sigmoid_prefill(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
                                              _p(head_bias), c_int(H), c_int(G), c_int(D), c_int(Dv), c_int(page), c_float(scale),
                                              c_int(chunk), c_int(window), _stream()), "attn_sigmoid_prefill")
     return out
+
+
+def gla_gate_decay(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None, tau: float, out: torch.Tensor) -> torch.Tensor:
+    """out[t, n] = sigmoid(sum_k x[t, k] w[n, k] + bias[n])^(1/tau), the sum and what follows in 32-bit. x [T, K] (a view
+    with unit inner stride), w [N, K] and bias [N] of one type, out float32 [T, N]."""
+    _gpu(x, w, bias, out)
+    T, K = x.shape
+    N = w.shape[0]
+    _need(x.stride(1) == 1 and w.is_contiguous() and tuple(w.shape) == (N, K) and w.dtype == x.dtype, f"gla_gate_decay: x [T, {K}], w [N, {K}] of one type")
+    if bias is not None:
+        _need(tuple(bias.shape) == (N,) and bias.is_contiguous() and bias.dtype == x.dtype, f"gla_gate_decay: bias [{N}] of x's type")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, N), f"gla_gate_decay: out float32 [{T}, {N}]")
+    _need(tau > 0, "gla_gate_decay: tau must be positive")
+    ldx = x.stride(0) if T > 1 else max(K, x.stride(0))
+    _check(library().tm_gla_gate_decay(_p(x), c_int(ldx), _p(w), _p(bias), c_int(code(x.dtype)), _p(out), c_int(T), c_int(N), c_int(K),
+                                       c_float(tau), _stream()), "gla_gate_decay")
+    return out
+
+
+def gla_segment_decay(decay: torch.Tensor, cu_seg: torch.Tensor, n_seg: int, out: torch.Tensor) -> torch.Tensor:
+    """out[c, j] = product over the rows cu_seg[c] .. cu_seg[c + 1] - 1 of decay[t, j]. decay float32 [T, HD]."""
+    _gpu(decay, cu_seg, out)
+    T, HD = decay.shape
+    _need(decay.dtype == torch.float32 and decay.is_contiguous(), "gla_segment_decay: decay is contiguous float32 [T, HD]")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (n_seg, HD), f"gla_segment_decay: out float32 [{n_seg}, {HD}]")
+    _ints(cu_seg, n_seg + 1, "cu_seg")
+    _need(n_seg <= 65535, "gla_segment_decay: at most 65,535 segments")
+    _check(library().tm_gla_segment_decay(_p(decay), _p(cu_seg), _p(out), c_int(n_seg), c_int(HD), _stream()), "gla_segment_decay")
+    return out
+
+
+def gla_combine(state: torch.Tensor, state_slots: torch.Tensor, first_seg: torch.Tensor, seg_decay: torch.Tensor,
+                local: torch.Tensor, start: torch.Tensor, num_seqs: int) -> None:
+    """For request s with segments first_seg[s] .. first_seg[s + 1] - 1: start[c] = B, B = diag(seg_decay[c]) B + local[c] in
+    their order, from B = state[state_slots[s]], which receives the last B. state [slots, H, D, Dv]; local, start
+    [n_seg, H, D, Dv]; seg_decay [n_seg, H * D]; all float32."""
+    _gpu(state, state_slots, first_seg, seg_decay, local, start)
+    n_seg = local.shape[0]
+    H, D, Dv = state.shape[1:]
+    for t, shape, name in ((state, None, "state"), (local, (n_seg, H, D, Dv), "local"), (start, (n_seg, H, D, Dv), "start"),
+                           (seg_decay, (n_seg, H * D), "seg_decay")):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and (shape is None or tuple(t.shape) == shape), f"gla_combine: {name} float32 {shape}")
+    _ints(state_slots, num_seqs, "state_slots")
+    _ints(first_seg, num_seqs + 1, "first_seg")
+    _need(num_seqs <= 65535, "gla_combine: at most 65,535 requests a step")
+    _check(library().tm_gla_combine(_p(state), _p(state_slots), _p(first_seg), _p(seg_decay), _p(local), _p(start), c_int(num_seqs),
+                                    c_int(H * D), c_int(Dv), _stream()), "gla_combine")

@@ -98,6 +98,9 @@ class GatedLinearAttention(Mixer):
             2 * seqs * self.num_heads * self.key_dim * self.value_dim * 4
         return moved, 4 * rows * self.num_heads * self.key_dim * self.value_dim
 
+    # Rows of a request's portion from which the recurrence runs in segments of this many rows (see ``_scan``)
+    SEGMENT = 64
+
     def forward(self, x, step: StepContext, cache: StateView, residual: torch.Tensor | None = None):
         x = as_tensor(x)
         T = x.shape[0]
@@ -105,13 +108,62 @@ class GatedLinearAttention(Mixer):
         ks, vs = self.k_size, self.v_size
         with profiling.label("qkv", lambda: self.cost("qkv", step, T)):
             proj = self.proj.forward(x)                                          # [T, q | k | v | g | a1]
-            decay = self.gate.forward(proj[:, 2 * ks + 2 * vs:], out_dtype=torch.float32)
-            ops.gla_decay(decay, self.tau)
+            narrow = proj[:, 2 * ks + 2 * vs:]
+            gate = self.gate
+            if gate.weight.dtype == narrow.dtype and (gate.bias is None or gate.bias.dtype == narrow.dtype):
+                decay = torch.empty((T, ks), dtype=torch.float32, device=x.device)
+                ops.gla_gate_decay(narrow, gate.weight, gate.bias, self.tau, decay)
+            else:                                                                # a matrix kept in another type: the product rule's way
+                decay = gate.forward(narrow, out_dtype=torch.float32)
+                ops.gla_decay(decay, self.tau)
         o = torch.empty((T, vs), dtype=torch.float32, device=x.device)
         y = torch.empty((T, vs), dtype=x.dtype, device=x.device)
-        with profiling.label("attention", lambda: self.cost("attention", step, T)):
-            ops.gla_scan(proj, 0, ks, 2 * ks, decay, o, cache.state, step.cu_q_lens, step.state_slots, step.num_seqs,
-                         H, D, Dv, D ** -0.5)
+        with profiling.label("recurrence", lambda: self.cost("attention", step, T)):
+            self._scan(proj, decay, o, cache.state, step)
             ops.gla_out_gate(o, proj[:, 2 * ks + vs:2 * ks + 2 * vs], self.norm_w, y, H, Dv, self.norm_eps)
         with profiling.label("o_proj", lambda: self.o.cost(T)):
             return self.o.forward(y)
+
+    def _scan(self, proj, decay, o, state, step: StepContext) -> None:
+        """The recurrence over the step's rows. A step whose longest portion is short (single tokens, small
+        portions) is one scan from the requests' states. A long portion is cut into segments of ``SEGMENT`` rows:
+        the recurrence is linear in the state, so every segment is first scanned from a zero state (what its own
+        rows build), a chain over the segments' decay products gives each segment's true start state and the
+        request's new state, and a second scan of all segments from those gives the results. Two scans that fill
+        the chip and a short chain, instead of one chain over every token. The sums of a token's result are then
+        ordered otherwise than in the plain chain: the two agree up to 32-bit rounding."""
+        H, D, Dv = self.num_heads, self.key_dim, self.value_dim
+        ks = self.k_size
+        scale = D ** -0.5
+        if step.max_q_len < 2 * self.SEGMENT:
+            ops.gla_scan(proj, 0, ks, 2 * ks, decay, o, state, step.cu_q_lens, step.state_slots, step.num_seqs, H, D, Dv, scale)
+            return
+        cu_seg, ids, first, n_seg = self._segments(step, proj.device)
+        local = torch.zeros((n_seg, H, D, Dv), dtype=torch.float32, device=proj.device)
+        ops.gla_scan(proj, 0, ks, 2 * ks, decay, o, local, cu_seg, ids, n_seg, H, D, Dv, scale)         # o: overwritten below
+        products = torch.empty((n_seg, ks), dtype=torch.float32, device=proj.device)
+        ops.gla_segment_decay(decay, cu_seg, n_seg, products)
+        start = torch.empty_like(local)
+        ops.gla_combine(state, step.state_slots, first, products, local, start, step.num_seqs)
+        ops.gla_scan(proj, 0, ks, 2 * ks, decay, o, start, cu_seg, ids, n_seg, H, D, Dv, scale)
+
+    def _segments(self, step: StepContext, device):
+        """(first row of each segment [n + 1], 0..n-1, first segment of each request [S + 1], n) on the device, made
+        once per step from the host's view of its portions and shared by the step's gla layers."""
+        made = getattr(step, "_gla_segments", None)
+        if made is None or made[0] != self.SEGMENT:
+            cu, first, row = [0], [0], 0
+            for n in step.q_lens:
+                for lo in range(0, n, self.SEGMENT):
+                    row += min(self.SEGMENT, n - lo)
+                    cu.append(row)
+                first.append(len(cu) - 1)
+            # q_lens covers the step's real requests; a step laid out in a padded shape is never segmented (its
+            # portions belong to a model without state)
+            if len(first) != step.num_seqs + 1 or row != step.num_tokens:
+                raise ValueError("the step's portions do not cover its rows: it cannot be cut into segments")
+            n_seg = len(cu) - 1
+            flat = torch.tensor(cu + list(range(n_seg)) + first, dtype=torch.int32).to(device)
+            made = (self.SEGMENT, flat[:n_seg + 1], flat[n_seg + 1:2 * n_seg + 1], flat[2 * n_seg + 1:], n_seg)
+            step._gla_segments = made
+        return made[1:]
