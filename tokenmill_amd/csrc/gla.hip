@@ -79,11 +79,135 @@ __global__ __launch_bounds__(TM_WAVE) void gla_scan_kernel(const T* __restrict__
         if (col && i < R && d0 + i < D) st[(size_t)(d0 + i) * Dv] = S[i];
 }
 
+// The same scan for sizes whose rows come in whole 16-byte pieces (D a multiple of 4 * 16 / sizeof(T), aligned rows): a
+// lane's R values of q, k and the decays are a few 16-byte loads instead of R small ones, and the next token's are
+// asked for before the current token is worked on. Same products and sums in the same order as the kernel above.
+template <typename T> struct Piece;
+template <> struct Piece<float> {
+    static constexpr int N = 4;
+    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+        f[0] = __uint_as_float(u.x); f[1] = __uint_as_float(u.y); f[2] = __uint_as_float(u.z); f[3] = __uint_as_float(u.w);
+    }
+};
+template <> struct Piece<bf16_t> {
+    static constexpr int N = 8;
+    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+        f[0] = __uint_as_float(u.x << 16); f[1] = __uint_as_float(u.x & 0xffff0000u);
+        f[2] = __uint_as_float(u.y << 16); f[3] = __uint_as_float(u.y & 0xffff0000u);
+        f[4] = __uint_as_float(u.z << 16); f[5] = __uint_as_float(u.z & 0xffff0000u);
+        f[6] = __uint_as_float(u.w << 16); f[7] = __uint_as_float(u.w & 0xffff0000u);
+    }
+};
+
+template <typename T, int RMAX>
+__global__ __launch_bounds__(TM_WAVE) void gla_scan_vec_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
+                                                              const float* __restrict__ decay, float* __restrict__ o,
+                                                              float* __restrict__ state, const int* __restrict__ cu_q_lens,
+                                                              const int* __restrict__ state_slots, int H, int D, int Dv,
+                                                              float q_scale) {
+    constexpr int EV = Piece<T>::N, NQ = RMAX / EV, NA = RMAX / 4;
+    const int lane = threadIdx.x, part = lane % GLA_PARTS;
+    const int e = blockIdx.x * GLA_COLS + lane / GLA_PARTS;
+    const int h = blockIdx.y, s = blockIdx.z;
+    const int R = D / GLA_PARTS;                      // a multiple of EV (and of 4): the host checks
+    const int nq = R / EV, na = R / 4;
+    const int d0 = part * R;
+    const bool col = e < Dv;
+    const int t0 = cu_q_lens[s], t1 = cu_q_lens[s + 1];
+    if (t1 <= t0) return;
+    float* st = state + (((size_t)state_slots[s] * H + h) * D) * Dv + (col ? e : 0);
+    float S[RMAX];
+#pragma unroll
+    for (int i = 0; i < RMAX; ++i) S[i] = (col && i < R) ? st[(size_t)(d0 + i) * Dv] : 0.f;
+    uint4 cq[NQ], ck[NQ], nq_[NQ], nk_[NQ];
+    float4 ca[NA], na_[NA];
+    float cv, nv;
+    const size_t head_q = (size_t)q_off + h * D + d0, head_k = (size_t)k_off + h * D + d0;
+    {
+        const T* row = proj + (size_t)t0 * ld;
+        const float* ar = decay + ((size_t)t0 * H + h) * D + d0;
+#pragma unroll
+        for (int i = 0; i < NQ; ++i)
+            if (i < nq) {
+                cq[i] = *(const uint4*)(row + head_q + i * EV);
+                ck[i] = *(const uint4*)(row + head_k + i * EV);
+            }
+#pragma unroll
+        for (int i = 0; i < NA; ++i)
+            if (i < na) ca[i] = *(const float4*)(ar + 4 * i);
+        cv = col ? Elem<T>::load(row + v_off + h * Dv + e) : 0.f;
+    }
+    for (int t = t0; t < t1; ++t) {
+        const int tn = t + 1 < t1 ? t + 1 : t;            // the last token asks for itself again
+        {
+            const T* row = proj + (size_t)tn * ld;
+            const float* ar = decay + ((size_t)tn * H + h) * D + d0;
+#pragma unroll
+            for (int i = 0; i < NQ; ++i)
+                if (i < nq) {
+                    nq_[i] = *(const uint4*)(row + head_q + i * EV);
+                    nk_[i] = *(const uint4*)(row + head_k + i * EV);
+                }
+#pragma unroll
+            for (int i = 0; i < NA; ++i)
+                if (i < na) na_[i] = *(const float4*)(ar + 4 * i);
+            nv = col ? Elem<T>::load(row + v_off + h * Dv + e) : 0.f;
+        }
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            if (i < nq) {
+                float qf[EV], kf[EV];
+                Piece<T>::unpack(cq[i], qf);
+                Piece<T>::unpack(ck[i], kf);
+#pragma unroll
+                for (int j = 0; j < EV; ++j) {
+                    const int r = i * EV + j;
+                    const float4 a4 = ca[r / 4];
+                    const float a = (r % 4 == 0) ? a4.x : (r % 4 == 1) ? a4.y : (r % 4 == 2) ? a4.z : a4.w;
+                    const float kv = kf[j] * cv;
+                    S[r] = a * S[r] + kv;
+                    acc += S[r] * (qf[j] * q_scale);
+                }
+            }
+        }
+        acc += __shfl_xor(acc, 1, TM_WAVE);
+        acc += __shfl_xor(acc, 2, TM_WAVE);
+        if (col && part == 0) o[((size_t)t * H + h) * Dv + e] = acc;
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) {
+            cq[i] = nq_[i];
+            ck[i] = nk_[i];
+        }
+#pragma unroll
+        for (int i = 0; i < NA; ++i) ca[i] = na_[i];
+        cv = nv;
+    }
+#pragma unroll
+    for (int i = 0; i < RMAX; ++i)
+        if (col && i < R) st[(size_t)(d0 + i) * Dv] = S[i];
+}
+
+template <typename T>
+static bool gla_scan_in_pieces(const void* proj, int ld, int q_off, int k_off, const float* decay, int D) {
+    constexpr int EV = Piece<T>::N;
+    return D % (GLA_PARTS * EV) == 0 && ld % EV == 0 && q_off % EV == 0 && k_off % EV == 0 && ((uintptr_t)proj % 16) == 0 &&
+           ((uintptr_t)decay % 16) == 0;
+}
+
 template <typename T>
 static int launch_gla_scan(const void* proj, int ld, int q_off, int k_off, int v_off, const float* decay, float* o, float* state,
                            const int* cu, const int* slots, int S, int H, int D, int Dv, float q_scale, hipStream_t stream) {
     const dim3 grid((Dv + GLA_COLS - 1) / GLA_COLS, H, S);
     const int R = (D + GLA_PARTS - 1) / GLA_PARTS;
+    if (R <= 32 && gla_scan_in_pieces<T>(proj, ld, q_off, k_off, decay, D)) {       // beyond 32 rows a lane the registers do not hold two tokens
+#define GLA_VEC(RM) gla_scan_vec_kernel<T, RM><<<grid, TM_WAVE, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu, slots, H, D, Dv, q_scale)
+        if (R <= 16) GLA_VEC(16);
+        else GLA_VEC(32);
+#undef GLA_VEC
+        TM_CHECK_LAUNCH();
+        return TM_OK;
+    }
     if (R <= 16)
         gla_scan_kernel<T, 16><<<grid, TM_WAVE, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu, slots, H,
                                                             D, Dv, q_scale);
