@@ -138,7 +138,7 @@ int tm_qk_norm_rope_store(void* qkv, int ld, int dtype, int T, int H, int G, int
 int tm_attn_sigmoid_paged(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
                           const int* block_tables, int table_width, const int* seq_of_token, const int* positions,
                           const float* head_bias, int T, int H, int G, int D, int Dv, int page, float scale, int chunk,
-                          int window, int dtype, hipStream_t stream);
+                          int window, int dtype, int split_keys, int n_splits, float* parts, hipStream_t stream);
 
 // The same attention for the prompt portions of a step on the matrix unit (attention_sigmoid_prefill.hip): bfloat16, the
 // step's tiles of up to 16 tokens as for tm_attn_prefill_mfma; tm_attn_sigmoid_prefill_takes says which sizes it runs.

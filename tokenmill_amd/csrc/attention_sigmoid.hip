@@ -106,7 +106,8 @@ __global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const T* __restrict__ k_pool,
     const T* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ seq_of_token, const int* __restrict__ positions, const float* __restrict__ head_bias, int H,
-    int G, int D, int Dv, int page, float scale, int chunk, int window) {
+    int G, int D, int Dv, int page, float scale, int chunk, int window, int split_keys, float* __restrict__ parts,
+    size_t part_stride) {
     extern __shared__ float lds[];
     float* qs = lds;                            // [D]
     float* wl = lds + D;                        // [64] weights of a round's keys
@@ -117,14 +118,21 @@ __global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_kernel(
     const int* tab = block_tables + (size_t)seq_of_token[t] * table_width;
     int lo = chunk > 0 ? (pos / chunk) * chunk : 0;
     if (window > 0 && pos - window + 1 > lo) lo = pos - window + 1;
+    // With `parts` the visible keys are dealt to blockIdx.z in runs of split_keys, counted from the first visible key, and
+    // the runs' sums go to parts[z] in 32-bit for the caller to add up in the order of z (a run without keys gives zeros).
+    int hi = pos;
+    if (parts) {
+        lo += (int)blockIdx.z * split_keys;
+        if (lo + split_keys - 1 < hi) hi = lo + split_keys - 1;
+    }
     const T* qr = q + (size_t)t * q_stride + (size_t)h * D;
     for (int d = lane; d < D; d += TM_WAVE) qs[d] = Elem<T>::load(qr + d);
     const float bias = head_bias ? head_bias[h] : 0.f;
     float acc[SG_MAX_DV / TM_WAVE] = {0.f, 0.f, 0.f, 0.f};
     __syncthreads();
-    for (int j0 = lo; j0 <= pos; j0 += TM_WAVE) {
+    for (int j0 = lo; j0 <= hi; j0 += TM_WAVE) {
         const int j = j0 + lane;
-        const bool valid = j <= pos;
+        const bool valid = j <= hi;
         const int pid = valid ? tab[j / page] : 0;
         float w = 0.f;
         if (valid) {
@@ -136,7 +144,7 @@ __global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_kernel(
         wl[lane] = w;
         pl[lane] = pid;
         __syncthreads();
-        const int n = min(TM_WAVE, pos - j0 + 1);
+        const int n = min(TM_WAVE, hi - j0 + 1);
 #pragma unroll
         for (int i = 0; i < SG_MAX_DV / TM_WAVE; ++i) {
             const int e = lane + TM_WAVE * i;
@@ -149,6 +157,15 @@ __global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_kernel(
         }
         __syncthreads();
     }
+    if (parts) {
+        float* po = parts + (size_t)blockIdx.z * part_stride + ((size_t)t * H + h) * Dv;
+#pragma unroll
+        for (int i = 0; i < SG_MAX_DV / TM_WAVE; ++i) {
+            const int e = lane + TM_WAVE * i;
+            if (e < Dv) po[e] = acc[i];
+        }
+        return;
+    }
     T* o = out + (size_t)t * out_stride + (size_t)h * Dv;
 #pragma unroll
     for (int i = 0; i < SG_MAX_DV / TM_WAVE; ++i) {
@@ -157,24 +174,30 @@ __global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_kernel(
     }
 }
 
+// n_splits > 0: the keys of every token in runs of split_keys over grid.z, 32-bit sums to parts [n_splits][T][H * Dv]
+// (`out` is not written; tm_sum_parts adds them up).
 extern "C" int tm_attn_sigmoid_paged(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                                      const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
                                      const int* positions, const float* head_bias, int T, int H, int G, int D, int Dv, int page,
-                                     float scale, int chunk, int window, int dtype, hipStream_t stream) {
+                                     float scale, int chunk, int window, int dtype, int split_keys, int n_splits, float* parts,
+                                     hipStream_t stream) {
     if (T <= 0) return TM_OK;
     if (H <= 0 || G <= 0 || H % G || D <= 0 || D > 256 || Dv <= 0 || Dv > SG_MAX_DV || page <= 0 || chunk < 0 || window < 0 ||
         table_width <= 0 || q_stride < H * D || out_stride < H * Dv || H > 65535)
         return TM_ERR_ARG;
-    const dim3 grid(T, H);
+    if (n_splits < 0 || n_splits > 65535 || (n_splits > 0 && (split_keys <= 0 || !parts))) return TM_ERR_ARG;
+    const dim3 grid(T, H, n_splits > 0 ? n_splits : 1);
+    float* pp = n_splits > 0 ? parts : nullptr;
+    const size_t part_stride = (size_t)T * H * Dv;
     const size_t lds = ((size_t)D + 2 * TM_WAVE) * sizeof(float);
     if (dtype == TM_F32)
         attn_sigmoid_paged_kernel<float><<<grid, TM_WAVE, lds, stream>>>(
             (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_pool, (const float*)v_pool, block_tables,
-            table_width, seq_of_token, positions, head_bias, H, G, D, Dv, page, scale, chunk, window);
+            table_width, seq_of_token, positions, head_bias, H, G, D, Dv, page, scale, chunk, window, split_keys, pp, part_stride);
     else if (dtype == TM_BF16)
         attn_sigmoid_paged_kernel<bf16_t><<<grid, TM_WAVE, lds, stream>>>(
             (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables,
-            table_width, seq_of_token, positions, head_bias, H, G, D, Dv, page, scale, chunk, window);
+            table_width, seq_of_token, positions, head_bias, H, G, D, Dv, page, scale, chunk, window, split_keys, pp, part_stride);
     else
         return TM_ERR_ARG;
     TM_CHECK_LAUNCH();

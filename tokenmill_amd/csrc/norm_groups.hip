@@ -43,29 +43,44 @@ __device__ __forceinline__ float group_scale(const float* part, int g, int split
     return 1.0f / sqrtf(ss / (float)glen + eps);
 }
 
-template <typename T, typename WT>
+// STAGE: the row of y and both weight vectors are copied into LDS beside the residual row by the first loop, so that
+// everything the block needs from memory is asked for at once (one trip instead of four dependent ones: a step of a
+// few rows is nothing but those trips); without it (rows too wide for that much LDS) they are read where they are used.
+template <typename T, typename WT, bool STAGE>
 __global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(float* __restrict__ resid, const T* __restrict__ y,
                                                                 const WT* __restrict__ post_w,
                                                                 const int* __restrict__ rows,
                                                                 const WT* __restrict__ pre_w, T* __restrict__ out,
                                                                 int hidden, int groups, int split, float eps) {
     extern __shared__ float lds[];
-    float* xs = lds;                    // the row, [hidden]
-    float* part = lds + hidden;         // [groups * split]
+    float* xs = lds;                                        // the row, [hidden]
+    float* ys = lds + hidden;                               // STAGE: y, post_w, pre_w, [hidden] each
+    float* pw = lds + 2 * hidden;
+    float* qw = lds + 3 * hidden;
+    float* part = lds + (STAGE ? 4 : 1) * hidden;           // [groups * split]
     const int r = blockIdx.x;
     const size_t src = rows ? (size_t)rows[r] : (size_t)r;
     float* x = resid + src * hidden;
+    const T* yr = y ? y + src * hidden : nullptr;
     const int glen = hidden / groups, units = groups * split;
-    for (int c = threadIdx.x; c < hidden; c += GN_THREADS) xs[c] = x[c];
-    if (y) {
-        const T* yr = y + src * hidden;
+    for (int c = threadIdx.x; c < hidden; c += GN_THREADS) {
+        xs[c] = x[c];
+        if (STAGE) {
+            if (yr) ys[c] = Elem<T>::load(yr + c);
+            if (post_w) pw[c] = Elem<WT>::load(post_w + c);
+            if (pre_w) qw[c] = Elem<WT>::load(pre_w + c);
+        }
+    }
+    if (STAGE) __syncthreads();
+    if (yr) {
         if (post_w) {
-            unit_sums([&](int c) { return Elem<T>::load(yr + c); }, part, glen, split, units);
+            if (STAGE) unit_sums([&](int c) { return ys[c]; }, part, glen, split, units);
+            else unit_sums([&](int c) { return Elem<T>::load(yr + c); }, part, glen, split, units);
             __syncthreads();
         }
         for (int c = threadIdx.x; c < hidden; c += GN_THREADS) {
-            float d = Elem<T>::load(yr + c);
-            if (post_w) d = Elem<WT>::load(post_w + c) * (d * group_scale(part, c / glen, split, glen, eps));
+            float d = STAGE ? ys[c] : Elem<T>::load(yr + c);
+            if (post_w) d = (STAGE ? pw[c] : Elem<WT>::load(post_w + c)) * (d * group_scale(part, c / glen, split, glen, eps));
             const float v = xs[c] + d;
             xs[c] = v;
             if (!rows) x[c] = v;
@@ -77,7 +92,20 @@ __global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(float* __restric
     __syncthreads();
     T* o = out + (size_t)r * hidden;
     for (int c = threadIdx.x; c < hidden; c += GN_THREADS)
-        Elem<T>::store(o + c, Elem<WT>::load(pre_w + c) * (xs[c] * group_scale(part, c / glen, split, glen, eps)));
+        Elem<T>::store(o + c, (STAGE ? qw[c] : Elem<WT>::load(pre_w + c)) * (xs[c] * group_scale(part, c / glen, split, glen, eps)));
+}
+
+template <typename T, typename WT>
+static void launch_group_norm(float* resid, const void* y, const void* post_w, const int* rows, const void* pre_w, void* out, int R,
+                              int hidden, int groups, int split, float eps, hipStream_t stream) {
+    const size_t units = (size_t)groups * split;
+    const size_t staged = (4 * (size_t)hidden + units) * sizeof(float), plain = ((size_t)hidden + units) * sizeof(float);
+    if (staged <= 64 * 1024)
+        group_norm_kernel<T, WT, true><<<R, GN_THREADS, staged, stream>>>(resid, (const T*)y, (const WT*)post_w, rows, (const WT*)pre_w,
+                                                                         (T*)out, hidden, groups, split, eps);
+    else
+        group_norm_kernel<T, WT, false><<<R, GN_THREADS, plain, stream>>>(resid, (const T*)y, (const WT*)post_w, rows, (const WT*)pre_w,
+                                                                         (T*)out, hidden, groups, split, eps);
 }
 
 extern "C" int tm_group_norm(float* resid, const void* y, const void* post_w, const int* rows, const void* pre_w,
@@ -91,17 +119,11 @@ extern "C" int tm_group_norm(float* resid, const void* y, const void* post_w, co
     const size_t lds = ((size_t)hidden + (size_t)groups * split) * sizeof(float);
     if (lds > 64 * 1024) return TM_ERR_ARG;
     if (dtype == TM_F32 && w_dtype == TM_F32)
-        group_norm_kernel<float, float><<<R, GN_THREADS, lds, stream>>>(resid, (const float*)y, (const float*)post_w, rows,
-                                                                       (const float*)pre_w, (float*)out, hidden, groups,
-                                                                       split, eps);
+        launch_group_norm<float, float>(resid, y, post_w, rows, pre_w, out, R, hidden, groups, split, eps, stream);
     else if (dtype == TM_BF16 && w_dtype == TM_BF16)
-        group_norm_kernel<bf16_t, bf16_t><<<R, GN_THREADS, lds, stream>>>(resid, (const bf16_t*)y, (const bf16_t*)post_w,
-                                                                         rows, (const bf16_t*)pre_w, (bf16_t*)out, hidden,
-                                                                         groups, split, eps);
+        launch_group_norm<bf16_t, bf16_t>(resid, y, post_w, rows, pre_w, out, R, hidden, groups, split, eps, stream);
     else if (dtype == TM_BF16 && w_dtype == TM_F32)
-        group_norm_kernel<bf16_t, float><<<R, GN_THREADS, lds, stream>>>(resid, (const bf16_t*)y, (const float*)post_w, rows,
-                                                                        (const float*)pre_w, (bf16_t*)out, hidden, groups,
-                                                                        split, eps);
+        launch_group_norm<bf16_t, float>(resid, y, post_w, rows, pre_w, out, R, hidden, groups, split, eps, stream);
     else
         return TM_ERR_ARG;
     TM_CHECK_LAUNCH();

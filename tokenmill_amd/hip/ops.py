@@ -1101,10 +1101,13 @@ def qk_norm_rope_store(qkv: torch.Tensor, H: int, G: int, D: int, Dv: int, q_w: 
 def attn_sigmoid_paged(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                        block_tables: torch.Tensor, seq_of_token: torch.Tensor, positions: torch.Tensor,
                        head_bias: torch.Tensor | None, H: int, G: int, D: int, Dv: int, scale: float, chunk: int = 0,
-                       window: int = 0) -> torch.Tensor:
+                       window: int = 0, split_keys: int = 0, most_keys: int = 0) -> torch.Tensor:
     """out[t, h] = sum over visible keys j of sigmoid(scale * q[t, h] . k[j] + head_bias[h]) * v[j]: every token of the step
     over its request's cache (its own key included), from the start of its chunk of ``chunk`` positions (0: from the
-    first) and at most ``window`` back (0: any). q [T, >= H*D] with unit inner stride, out [T, H*Dv]."""
+    first) and at most ``window`` back (0: any). q [T, >= H*D] with unit inner stride, out [T, H*Dv].
+    ``split_keys`` > 0: a token's visible keys are dealt in runs of that many (counted from its first visible key) to
+    ceil(most_keys / split_keys) wavefronts whose 32-bit sums are added in their order; ``most_keys``: the most keys any
+    token of the call sees. Few tokens with long contexts then fill the chip."""
     _gpu(q, out, k_pool, v_pool, block_tables, seq_of_token, positions, head_bias)
     T = q.shape[0]
     _need(q.stride(1) == 1 and q.shape[1] >= H * D and out.is_contiguous() and tuple(out.shape) == (T, H * Dv),
@@ -1121,10 +1124,19 @@ def attn_sigmoid_paged(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor,
               f"attention(sigmoid): head_bias is float32 [{H}]")
     _need(chunk >= 0 and window >= 0, "attention(sigmoid): chunk and window must be >= 0")
     q_stride = q.stride(0) if T > 1 else max(q.stride(0), H * D)
+    n_splits, parts = 0, None
+    if split_keys > 0 and T > 0:
+        _need(most_keys > 0, "attention(sigmoid): split keys need the most keys a token sees")
+        n_splits = -(-most_keys // split_keys)
+        _need(n_splits <= 65535, "attention(sigmoid): too many runs of keys")
+        parts = torch.empty((n_splits, T, H * Dv), dtype=torch.float32, device=q.device)
     _check(library().tm_attn_sigmoid_paged(_p(q), c_int(q_stride), _p(out), c_int(H * Dv), _p(k_pool), _p(v_pool), _p(block_tables),
                                            c_int(block_tables.shape[1]), _p(seq_of_token), _p(positions), _p(head_bias), c_int(T),
                                            c_int(H), c_int(G), c_int(D), c_int(Dv), c_int(page), c_float(scale), c_int(chunk),
-                                           c_int(window), c_int(code(q.dtype)), _stream()), "attn_sigmoid_paged")
+                                           c_int(window), c_int(code(q.dtype)), c_int(split_keys if n_splits else 0), c_int(n_splits),
+                                           _p(parts), _stream()), "attn_sigmoid_paged")
+    if parts is not None:
+        sum_parts(parts, out)
     return out
 
 

@@ -25,6 +25,8 @@ MAX_HEAD_DIM = 256
 
 
 class SigmoidAttention(Mixer):
+    SPLIT_KEYS = 256        # keys of a single token that one wavefront sums; more are dealt to several
+
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int, scale: float,
                  rotary: RotaryEmbedding | None = None, qk_norm_eps: float | None = None, head_bias: bool = True,
                  chunk: int | None = None, window: int | None = None,
@@ -141,5 +143,15 @@ class SigmoidAttention(Mixer):
             rows = slice(first_single, T)
         else:
             rows = slice(0, T)
+        # Single tokens are few and may see many keys: where the model lets a token see more than SPLIT_KEYS of them, its
+        # keys are dealt in runs of that many to wavefronts of their own (whether they are is the model's matter, not
+        # the step's, so a token's sums have one order whatever it is batched with; a run beyond a token's keys adds zeros)
+        split = most = 0
+        if rows.start == first_single and step.num_decode > 0:
+            bound = min(x for x in (self.chunk, self.window, self.rotary.max_positions if self.rotary is not None else None, 1 << 30)
+                        if x is not None)
+            if bound > self.SPLIT_KEYS:
+                split, most = self.SPLIT_KEYS, max(1, min(bound, step.max_decode_context))
         ops.attn_sigmoid_paged(qkv[rows], out[rows], cache.k, cache.v, group.block_tables, step.seq_of_token[rows],
-                               step.positions[rows], self.head_bias, H, G, D, Dv, self.scale, self.chunk or 0, self.window or 0)
+                               step.positions[rows], self.head_bias, H, G, D, Dv, self.scale, self.chunk or 0, self.window or 0,
+                               split_keys=split, most_keys=most)
