@@ -138,7 +138,8 @@ __global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_kernel(
         if (valid) {
             const T* kr = k_pool + (((size_t)pid * page + j % page) * G + g) * D;
             float s = 0.f;
-            for (int d = 0; d < D; ++d) s += qs[d] * Elem<T>::load(kr + d);
+#pragma unroll 16
+            for (int d = 0; d < D; ++d) s += qs[d] * Elem<T>::load(kr + d);       // sixteen loads in flight, added in ascending d
             w = sigmoid_f32(s * scale + bias);
         }
         wl[lane] = w;
@@ -150,6 +151,7 @@ __global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_kernel(
             const int e = lane + TM_WAVE * i;
             if (e < Dv) {
                 float a = acc[i];
+#pragma unroll 16
                 for (int jj = 0; jj < n; ++jj)
                     a += wl[jj] * Elem<T>::load(v_pool + (((size_t)pl[jj] * G + g) * Dv + e) * page + (j0 + jj) % page);
                 acc[i] = a;

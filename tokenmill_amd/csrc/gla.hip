@@ -284,6 +284,7 @@ __global__ __launch_bounds__(256) void gla_gate_decay_kernel(const T* __restrict
     const T* xr = x + (size_t)t * ldx;
     const T* wr = W + (size_t)n * K;
     float z = bias ? Elem<T>::load(bias + n) : 0.f;
+#pragma unroll 16
     for (int k = 0; k < K; ++k) z += Elem<T>::load(xr + k) * Elem<T>::load(wr + k);
     const float ls = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
     a[(size_t)t * N + n] = expf(ls * inv_tau);

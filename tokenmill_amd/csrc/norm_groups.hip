@@ -28,6 +28,7 @@ __device__ __forceinline__ void unit_sums(Load at, float* part, int glen, int sp
         const int lo = g * glen + i * plen;
         const int hi = min(lo + plen, (g + 1) * glen);
         float ss = 0.f;
+#pragma unroll 8
         for (int c = lo + lane; c < hi; c += TM_WAVE) {
             const float x = at(c);
             ss += x * x;
@@ -37,10 +38,15 @@ __device__ __forceinline__ void unit_sums(Load at, float* part, int glen, int sp
     }
 }
 
-__device__ __forceinline__ float group_scale(const float* part, int g, int split, int glen, float eps) {
-    float ss = part[g * split];
-    for (int i = 1; i < split; ++i) ss += part[g * split + i];
-    return 1.0f / sqrtf(ss / (float)glen + eps);
+// The groups' 1 / sqrt(mean + eps) from their units' sums, once per group (a root and two divisions per element
+// were most of a small step's time), into scale[groups]. Ends with a barrier.
+__device__ __forceinline__ void group_scales(const float* part, float* scale, int groups, int split, int glen, float eps) {
+    for (int g = threadIdx.x; g < groups; g += GN_THREADS) {
+        float ss = part[g * split];
+        for (int i = 1; i < split; ++i) ss += part[g * split + i];
+        scale[g] = 1.0f / sqrtf(ss / (float)glen + eps);
+    }
+    __syncthreads();
 }
 
 // STAGE: the row of y and both weight vectors are copied into LDS beside the residual row by the first loop, so that
@@ -58,11 +64,14 @@ __global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(float* __restric
     float* pw = lds + 2 * hidden;
     float* qw = lds + 3 * hidden;
     float* part = lds + (STAGE ? 4 : 1) * hidden;           // [groups * split]
+    float* scale = part + groups * split;                   // [groups]
     const int r = blockIdx.x;
     const size_t src = rows ? (size_t)rows[r] : (size_t)r;
     float* x = resid + src * hidden;
     const T* yr = y ? y + src * hidden : nullptr;
     const int glen = hidden / groups, units = groups * split;
+    // unrolled: the loads of eight rounds are in flight together (left as a loop, every round waits for its own)
+#pragma unroll 8
     for (int c = threadIdx.x; c < hidden; c += GN_THREADS) {
         xs[c] = x[c];
         if (STAGE) {
@@ -77,10 +86,12 @@ __global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(float* __restric
             if (STAGE) unit_sums([&](int c) { return ys[c]; }, part, glen, split, units);
             else unit_sums([&](int c) { return Elem<T>::load(yr + c); }, part, glen, split, units);
             __syncthreads();
+            group_scales(part, scale, groups, split, glen, eps);
         }
+#pragma unroll 8
         for (int c = threadIdx.x; c < hidden; c += GN_THREADS) {
             float d = STAGE ? ys[c] : Elem<T>::load(yr + c);
-            if (post_w) d = (STAGE ? pw[c] : Elem<WT>::load(post_w + c)) * (d * group_scale(part, c / glen, split, glen, eps));
+            if (post_w) d = (STAGE ? pw[c] : Elem<WT>::load(post_w + c)) * (d * scale[c / glen]);
             const float v = xs[c] + d;
             xs[c] = v;
             if (!rows) x[c] = v;
@@ -90,15 +101,17 @@ __global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(float* __restric
     __syncthreads();
     unit_sums([&](int c) { return xs[c]; }, part, glen, split, units);
     __syncthreads();
+    group_scales(part, scale, groups, split, glen, eps);
     T* o = out + (size_t)r * hidden;
+#pragma unroll 8
     for (int c = threadIdx.x; c < hidden; c += GN_THREADS)
-        Elem<T>::store(o + c, (STAGE ? qw[c] : Elem<WT>::load(pre_w + c)) * (xs[c] * group_scale(part, c / glen, split, glen, eps)));
+        Elem<T>::store(o + c, (STAGE ? qw[c] : Elem<WT>::load(pre_w + c)) * (xs[c] * scale[c / glen]));
 }
 
 template <typename T, typename WT>
 static void launch_group_norm(float* resid, const void* y, const void* post_w, const int* rows, const void* pre_w, void* out, int R,
                               int hidden, int groups, int split, float eps, hipStream_t stream) {
-    const size_t units = (size_t)groups * split;
+    const size_t units = (size_t)groups * split + groups;       // the units' sums and the groups' scales
     const size_t staged = (4 * (size_t)hidden + units) * sizeof(float), plain = ((size_t)hidden + units) * sizeof(float);
     if (staged <= 64 * 1024)
         group_norm_kernel<T, WT, true><<<R, GN_THREADS, staged, stream>>>(resid, (const T*)y, (const WT*)post_w, rows, (const WT*)pre_w,
@@ -116,7 +129,7 @@ extern "C" int tm_group_norm(float* resid, const void* y, const void* post_w, co
     if ((out == nullptr) != (pre_w == nullptr)) return TM_ERR_ARG;
     if (!y && post_w) return TM_ERR_ARG;
     const int split = groups >= GN_WAVES ? 1 : GN_WAVES / groups;
-    const size_t lds = ((size_t)hidden + (size_t)groups * split) * sizeof(float);
+    const size_t lds = ((size_t)hidden + (size_t)groups * split + groups) * sizeof(float);
     if (lds > 64 * 1024) return TM_ERR_ARG;
     if (dtype == TM_F32 && w_dtype == TM_F32)
         launch_group_norm<float, float>(resid, y, post_w, rows, pre_w, out, R, hidden, groups, split, eps, stream);

@@ -1026,7 +1026,7 @@ def group_norm(resid: torch.Tensor, y: torch.Tensor | None, post_w: torch.Tensor
     R = T if rows is None else rows.numel()
     _need(resid.dtype == torch.float32 and resid.is_contiguous(), "group_norm: the residual stream is contiguous float32")
     _need(groups >= 1 and hidden % groups == 0, f"group_norm: {groups} groups do not divide the width {hidden}")
-    _need(hidden + 4 * groups <= GROUP_NORM_MAX_FLOATS, f"group_norm: a row of {hidden} does not fit the kernel's LDS")
+    _need(hidden + 5 * groups <= GROUP_NORM_MAX_FLOATS, f"group_norm: a row of {hidden} does not fit the kernel's LDS")
     _need((out is None) == (pre_w is None), "group_norm: out and its norm's weight come together")
     _need(post_w is None or y is not None, "group_norm: a norm of y needs y")
     dtype = out.dtype if out is not None else y.dtype if y is not None else None
