@@ -176,6 +176,114 @@ __global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_kernel(
     }
 }
 
+// The same kernel for sizes whose key rows and pages come in whole 16-byte pieces (D and the page size multiples of
+// 16 / sizeof(T)): a key's row is read by eight lanes in 16-byte pieces (eight keys a step, all of a round's loads
+// in flight at once) and a value channel reads its keys 16 bytes at a time, so a round is a few trips to memory instead
+// of a hundred small dependent ones. The scores' sums are ordered otherwise than in the kernel above (a lane's pieces in
+// ascending order, then the eight lanes by a fixed tree); which of the two kernels runs follows from the model's sizes.
+template <typename T>
+__global__ __launch_bounds__(TM_WAVE) void attn_sigmoid_paged_vec_kernel(
+    const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const T* __restrict__ k_pool,
+    const T* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
+    const int* __restrict__ seq_of_token, const int* __restrict__ positions, const float* __restrict__ head_bias, int H,
+    int G, int D, int Dv, int page, float scale, int chunk, int window, int split_keys, float* __restrict__ parts,
+    size_t part_stride) {
+    constexpr int EV = Piece<T>::N;
+    extern __shared__ float lds[];
+    float* qs = lds;                            // [D]
+    float* wl = lds + D;                        // [64] weights of a round's keys
+    int* pl = (int*)(lds + D + TM_WAVE);        // [64] their pages
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int g = h / (H / G);
+    const int pos = positions[t];
+    const int* tab = block_tables + (size_t)seq_of_token[t] * table_width;
+    int lo = chunk > 0 ? (pos / chunk) * chunk : 0;
+    if (window > 0 && pos - window + 1 > lo) lo = pos - window + 1;
+    int hi = pos;
+    if (parts) {
+        lo += (int)blockIdx.z * split_keys;
+        if (lo + split_keys - 1 < hi) hi = lo + split_keys - 1;
+    }
+    const T* qr = q + (size_t)t * q_stride + (size_t)h * D;
+    for (int d = lane; d < D; d += TM_WAVE) qs[d] = Elem<T>::load(qr + d);
+    const float bias = head_bias ? head_bias[h] : 0.f;
+    float acc[SG_MAX_DV / TM_WAVE] = {0.f, 0.f, 0.f, 0.f};
+    const int kk = lane / 8, piece = lane % 8;  // eight lanes a key, eight keys a step
+    const int np = D / EV;
+    __syncthreads();
+    for (int j0 = lo; j0 <= hi; j0 += TM_WAVE) {
+#pragma unroll
+        for (int ss = 0; ss < 8; ++ss) {
+            const int jj = ss * 8 + kk, j = j0 + jj;
+            const bool valid = j <= hi;
+            const int pid = valid ? tab[j / page] : 0;
+            float part = 0.f;
+            if (valid) {
+                const T* kr = k_pool + (((size_t)pid * page + j % page) * G + g) * D;
+                for (int p = piece; p < np; p += 8) {
+                    float kf[EV];
+                    Piece<T>::unpack(*(const uint4*)(kr + p * EV), kf);
+#pragma unroll
+                    for (int i = 0; i < EV; ++i) part += qs[p * EV + i] * kf[i];
+                }
+            }
+            part += __shfl_xor(part, 1, TM_WAVE);
+            part += __shfl_xor(part, 2, TM_WAVE);
+            part += __shfl_xor(part, 4, TM_WAVE);
+            if (piece == 0) {
+                wl[jj] = valid ? sigmoid_f32(part * scale + bias) : 0.f;
+                pl[jj] = pid;
+            }
+        }
+        __syncthreads();
+        const int n = min(TM_WAVE, hi - j0 + 1);
+        const int head = min(n, (EV - j0 % EV) % EV);       // keys before the first that starts a 16-byte piece
+        const int pieces = (n - head) / EV;
+#pragma unroll
+        for (int i = 0; i < SG_MAX_DV / TM_WAVE; ++i) {
+            const int e = lane + TM_WAVE * i;
+            if (e < Dv) {
+                float a = acc[i];
+                int jj = 0;
+                for (; jj < head; ++jj)
+                    a += wl[jj] * Elem<T>::load(v_pool + (((size_t)pl[jj] * G + g) * Dv + e) * page + (j0 + jj) % page);
+#pragma unroll 4
+                for (int pc = 0; pc < pieces; ++pc, jj += EV) {
+                    float vf[EV];
+                    Piece<T>::unpack(*(const uint4*)(v_pool + (((size_t)pl[jj] * G + g) * Dv + e) * page + (j0 + jj) % page), vf);
+#pragma unroll
+                    for (int k = 0; k < EV; ++k) a += wl[jj + k] * vf[k];
+                }
+                for (; jj < n; ++jj)
+                    a += wl[jj] * Elem<T>::load(v_pool + (((size_t)pl[jj] * G + g) * Dv + e) * page + (j0 + jj) % page);
+                acc[i] = a;
+            }
+        }
+        __syncthreads();
+    }
+    if (parts) {
+        float* po = parts + (size_t)blockIdx.z * part_stride + ((size_t)t * H + h) * Dv;
+#pragma unroll
+        for (int i = 0; i < SG_MAX_DV / TM_WAVE; ++i) {
+            const int e = lane + TM_WAVE * i;
+            if (e < Dv) po[e] = acc[i];
+        }
+        return;
+    }
+    T* o = out + (size_t)t * out_stride + (size_t)h * Dv;
+#pragma unroll
+    for (int i = 0; i < SG_MAX_DV / TM_WAVE; ++i) {
+        const int e = lane + TM_WAVE * i;
+        if (e < Dv) Elem<T>::store(o + e, acc[i]);
+    }
+}
+
+template <typename T>
+static bool sigmoid_in_pieces(const void* k_pool, const void* v_pool, int D, int page) {
+    constexpr int EV = Piece<T>::N;
+    return D % EV == 0 && page % EV == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0;
+}
+
 // n_splits > 0: the keys of every token in runs of split_keys over grid.z, 32-bit sums to parts [n_splits][T][H * Dv]
 // (`out` is not written; tm_sum_parts adds them up).
 extern "C" int tm_attn_sigmoid_paged(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
@@ -192,7 +300,15 @@ extern "C" int tm_attn_sigmoid_paged(const void* q, int q_stride, void* out, int
     float* pp = n_splits > 0 ? parts : nullptr;
     const size_t part_stride = (size_t)T * H * Dv;
     const size_t lds = ((size_t)D + 2 * TM_WAVE) * sizeof(float);
-    if (dtype == TM_F32)
+    if (dtype == TM_F32 && sigmoid_in_pieces<float>(k_pool, v_pool, D, page))
+        attn_sigmoid_paged_vec_kernel<float><<<grid, TM_WAVE, lds, stream>>>(
+            (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_pool, (const float*)v_pool, block_tables,
+            table_width, seq_of_token, positions, head_bias, H, G, D, Dv, page, scale, chunk, window, split_keys, pp, part_stride);
+    else if (dtype == TM_BF16 && sigmoid_in_pieces<bf16_t>(k_pool, v_pool, D, page))
+        attn_sigmoid_paged_vec_kernel<bf16_t><<<grid, TM_WAVE, lds, stream>>>(
+            (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables,
+            table_width, seq_of_token, positions, head_bias, H, G, D, Dv, page, scale, chunk, window, split_keys, pp, part_stride);
+    else if (dtype == TM_F32)
         attn_sigmoid_paged_kernel<float><<<grid, TM_WAVE, lds, stream>>>(
             (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_pool, (const float*)v_pool, block_tables,
             table_width, seq_of_token, positions, head_bias, H, G, D, Dv, page, scale, chunk, window, split_keys, pp, part_stride);

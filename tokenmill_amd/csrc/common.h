@@ -43,6 +43,24 @@ template <> struct Elem<bf16_t> {
     static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 };
 
+// Sixteen bytes of a row as 32-bit floats: 4 float32 values or 8 bfloat16 values.
+template <typename T> struct Piece;
+template <> struct Piece<float> {
+    static constexpr int N = 4;
+    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+        f[0] = __uint_as_float(u.x); f[1] = __uint_as_float(u.y); f[2] = __uint_as_float(u.z); f[3] = __uint_as_float(u.w);
+    }
+};
+template <> struct Piece<bf16_t> {
+    static constexpr int N = 8;
+    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+        f[0] = __uint_as_float(u.x << 16); f[1] = __uint_as_float(u.x & 0xffff0000u);
+        f[2] = __uint_as_float(u.y << 16); f[3] = __uint_as_float(u.y & 0xffff0000u);
+        f[4] = __uint_as_float(u.z << 16); f[5] = __uint_as_float(u.z & 0xffff0000u);
+        f[6] = __uint_as_float(u.w << 16); f[7] = __uint_as_float(u.w & 0xffff0000u);
+    }
+};
+
 // The rotation of a pair (x1, x2) by the angle whose cosine and sine are c and s (reference
 // src/infer/model/layers.py:60-64). Every product and each sum is rounded to 32-bit on its own, as a tensor
 // library's x1 * cos - x2 * sin is: left to itself the compiler fuses a product into the sum, and which one it

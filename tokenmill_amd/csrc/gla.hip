@@ -82,23 +82,6 @@ __global__ __launch_bounds__(TM_WAVE) void gla_scan_kernel(const T* __restrict__
 // The same scan for sizes whose rows come in whole 16-byte pieces (D a multiple of 4 * 16 / sizeof(T), aligned rows): a
 // lane's R values of q, k and the decays are a few 16-byte loads instead of R small ones, and the next token's are
 // asked for before the current token is worked on. Same products and sums in the same order as the kernel above.
-template <typename T> struct Piece;
-template <> struct Piece<float> {
-    static constexpr int N = 4;
-    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
-        f[0] = __uint_as_float(u.x); f[1] = __uint_as_float(u.y); f[2] = __uint_as_float(u.z); f[3] = __uint_as_float(u.w);
-    }
-};
-template <> struct Piece<bf16_t> {
-    static constexpr int N = 8;
-    static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
-        f[0] = __uint_as_float(u.x << 16); f[1] = __uint_as_float(u.x & 0xffff0000u);
-        f[2] = __uint_as_float(u.y << 16); f[3] = __uint_as_float(u.y & 0xffff0000u);
-        f[4] = __uint_as_float(u.z << 16); f[5] = __uint_as_float(u.z & 0xffff0000u);
-        f[6] = __uint_as_float(u.w << 16); f[7] = __uint_as_float(u.w & 0xffff0000u);
-    }
-};
-
 template <typename T, int RMAX>
 __global__ __launch_bounds__(TM_WAVE) void gla_scan_vec_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
                                                               const float* __restrict__ decay, float* __restrict__ o,
