@@ -108,9 +108,146 @@ __global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(float* __restric
         Elem<T>::store(o + c, (STAGE ? qw[c] : Elem<WT>::load(pre_w + c)) * (xs[c] * scale[c / glen]));
 }
 
+// The same operation with a row in registers, for rows of at most 4,096 elements in whole groups of four and at most
+// eight groups: a thread keeps its (up to four) 4-element pieces of x, y and both weights, which it asked for at once;
+// the groups' sums of squares go lane to lane and then through LDS, one barrier per norm. A decode step's norm is a
+// chain of dependent steps at a low clock: this one is a third as long as the kernel above.
+#define GN_MAX_GROUPS 8
+#define GN_PIECES 4
+
+typedef float gn_f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct GnVec;
+template <> struct GnVec<float> {
+    static __device__ __forceinline__ gn_f32x4 load(const float* p) { return *(const gn_f32x4*)p; }
+    static __device__ __forceinline__ void store(float* p, gn_f32x4 v) { *(gn_f32x4*)p = v; }
+};
+template <> struct GnVec<bf16_t> {
+    static __device__ __forceinline__ gn_f32x4 load(const bf16_t* p) {
+        const uint2 u = *(const uint2*)p;
+        return gn_f32x4{__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                        __uint_as_float(u.y & 0xffff0000u)};
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, gn_f32x4 v) {
+        uint2 u;
+        u.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        u.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        *(uint2*)p = u;
+    }
+};
+
+// 1 / sqrt(mean + eps) of every group from the threads' per-piece sums of squares; sums[i] belongs to group grp[i]
+// (-1: no piece). Every thread gets all groups' scales. Lanes are added by the fixed tree of wave_sum, wavefronts in order.
+__device__ __forceinline__ void gn_scales(const float (&sums)[GN_PIECES], const int (&grp)[GN_PIECES], int groups, int glen,
+                                          float eps, float* red /* [GN_WAVES][GN_MAX_GROUPS] */, float (&scale)[GN_MAX_GROUPS]) {
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+    float mine[GN_MAX_GROUPS];
+#pragma unroll
+    for (int k = 0; k < GN_MAX_GROUPS; ++k) {
+        float v = 0.f;
+#pragma unroll
+        for (int i = 0; i < GN_PIECES; ++i)
+            if (grp[i] == k) v += sums[i];
+        mine[k] = k < groups ? wave_sum(v) : 0.f;
+    }
+    __syncthreads();                            // the last use of red is over
+    if (lane == 0) {
+#pragma unroll
+        for (int k = 0; k < GN_MAX_GROUPS; ++k) red[wave * GN_MAX_GROUPS + k] = mine[k];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < GN_MAX_GROUPS; ++k) {
+        float ss = red[k];
+#pragma unroll
+        for (int w = 1; w < GN_WAVES; ++w) ss += red[w * GN_MAX_GROUPS + k];
+        scale[k] = k < groups ? 1.0f / sqrtf(ss / (float)glen + eps) : 0.f;
+    }
+}
+
+template <typename T, typename WT>
+__global__ __launch_bounds__(GN_THREADS) void group_norm_reg_kernel(float* __restrict__ resid, const T* __restrict__ y,
+                                                                    const WT* __restrict__ post_w, const int* __restrict__ rows,
+                                                                    const WT* __restrict__ pre_w, T* __restrict__ out,
+                                                                    int hidden, int groups, float eps) {
+    __shared__ float red[GN_WAVES * GN_MAX_GROUPS];
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* x = resid + src * hidden;
+    const T* yr = y ? y + src * hidden : nullptr;
+    const int glen = hidden / groups, pieces = hidden / 4;
+    gn_f32x4 xv[GN_PIECES], yv[GN_PIECES], pw[GN_PIECES], qw[GN_PIECES];
+    int grp[GN_PIECES];
+#pragma unroll
+    for (int i = 0; i < GN_PIECES; ++i) {
+        const int pc = threadIdx.x + i * GN_THREADS;
+        grp[i] = -1;
+        xv[i] = yv[i] = pw[i] = qw[i] = gn_f32x4{0.f, 0.f, 0.f, 0.f};
+        if (pc < pieces) {
+            grp[i] = 4 * pc / glen;             // a piece lies in one group (glen % 4 == 0)
+            xv[i] = GnVec<float>::load(x + 4 * pc);
+            if (yr) yv[i] = GnVec<T>::load(yr + 4 * pc);
+            if (post_w) pw[i] = GnVec<WT>::load(post_w + 4 * pc);
+            if (pre_w) qw[i] = GnVec<WT>::load(pre_w + 4 * pc);
+        }
+    }
+    float sums[GN_PIECES], scale[GN_MAX_GROUPS];
+    if (yr) {
+        if (post_w) {
+#pragma unroll
+            for (int i = 0; i < GN_PIECES; ++i)
+                sums[i] = yv[i][0] * yv[i][0] + yv[i][1] * yv[i][1] + yv[i][2] * yv[i][2] + yv[i][3] * yv[i][3];
+            gn_scales(sums, grp, groups, glen, eps, red, scale);
+        }
+#pragma unroll
+        for (int i = 0; i < GN_PIECES; ++i) {
+            if (grp[i] < 0) continue;
+            float sc = 1.f;
+            if (post_w) {
+#pragma unroll
+                for (int k = 0; k < GN_MAX_GROUPS; ++k)
+                    if (grp[i] == k) sc = scale[k];
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) xv[i][k] += post_w ? pw[i][k] * (yv[i][k] * sc) : yv[i][k];
+            if (!rows) GnVec<float>::store(x + 4 * (threadIdx.x + i * GN_THREADS), xv[i]);
+        }
+    }
+    if (!out) return;
+#pragma unroll
+    for (int i = 0; i < GN_PIECES; ++i)
+        sums[i] = xv[i][0] * xv[i][0] + xv[i][1] * xv[i][1] + xv[i][2] * xv[i][2] + xv[i][3] * xv[i][3];
+    gn_scales(sums, grp, groups, glen, eps, red, scale);
+    T* o = out + (size_t)r * hidden;
+#pragma unroll
+    for (int i = 0; i < GN_PIECES; ++i) {
+        if (grp[i] < 0) continue;
+        float sc = 1.f;
+#pragma unroll
+        for (int k = 0; k < GN_MAX_GROUPS; ++k)
+            if (grp[i] == k) sc = scale[k];
+        gn_f32x4 v;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) v[k] = qw[i][k] * (xv[i][k] * sc);
+        GnVec<T>::store(o + 4 * (threadIdx.x + i * GN_THREADS), v);
+    }
+}
+
+static bool gn_in_registers(const float* resid, const void* y, const void* post_w, const void* pre_w, const void* out, int hidden,
+                            int groups, int elem, int w_elem) {
+    auto ok = [](const void* p, int bytes) { return !p || ((uintptr_t)p % bytes) == 0; };
+    return hidden % 4 == 0 && hidden <= 4 * GN_THREADS * GN_PIECES && groups <= GN_MAX_GROUPS && (hidden / groups) % 4 == 0 &&
+           ok(resid, 16) && ok(y, 4 * elem) && ok(out, 4 * elem) && ok(post_w, 4 * w_elem) && ok(pre_w, 4 * w_elem);
+}
+
 template <typename T, typename WT>
 static void launch_group_norm(float* resid, const void* y, const void* post_w, const int* rows, const void* pre_w, void* out, int R,
                               int hidden, int groups, int split, float eps, hipStream_t stream) {
+    if (gn_in_registers(resid, y, post_w, pre_w, out, hidden, groups, (int)sizeof(T), (int)sizeof(WT))) {
+        group_norm_reg_kernel<T, WT><<<R, GN_THREADS, 0, stream>>>(resid, (const T*)y, (const WT*)post_w, rows, (const WT*)pre_w,
+                                                                  (T*)out, hidden, groups, eps);
+        return;
+    }
     const size_t units = (size_t)groups * split + groups;       // the units' sums and the groups' scales
     const size_t staged = (4 * (size_t)hidden + units) * sizeof(float), plain = ((size_t)hidden + units) * sizeof(float);
     if (staged <= 64 * 1024)
