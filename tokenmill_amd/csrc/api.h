@@ -153,6 +153,8 @@ int tm_gla_decay(const float* z, float* a, float tau, long long n, hipStream_t s
 int tm_gla_scan(const void* proj, int ld, int q_off, int k_off, int v_off, int dtype, const float* decay, float* o,
                 float* state, const int* cu_q_lens, const int* state_slots, int S, int H, int D, int Dv, float q_scale,
                 hipStream_t stream);
+// Whether tm_gla_scan takes o == nullptr for these operands (only the states are advanced): rows in whole 16-byte pieces.
+int tm_gla_scan_in_pieces(int dtype, const void* proj, int ld, int q_off, int k_off, const float* decay, int D);
 int tm_gla_out_gate(const float* o, const void* gate, int ldg, int dtype, const float* w, void* y, int T, int H, int Dv,
                     float eps, hipStream_t stream);
 // The decays straight from the narrow projection x [T, K] (rows ldx apart), W [N, K], bias [N] of the model's type:

@@ -82,17 +82,19 @@ __global__ __launch_bounds__(TM_WAVE) void gla_scan_kernel(const T* __restrict__
 // The same scan for sizes whose rows come in whole 16-byte pieces (D a multiple of 4 * 16 / sizeof(T), aligned rows): a
 // lane's R values of q, k and the decays are a few 16-byte loads instead of R small ones, and the next token's are
 // asked for before the current token is worked on. Same products and sums in the same order as the kernel above.
-template <typename T, int RMAX>
+// PARTS lanes share a column's rows (4 or 8: with 8, a lane holds half as much and twice as many wavefronts hide each
+// other's loads); OUT = false leaves q and the results out (the scan that only builds the segments' local states).
+template <typename T, int RMAX, int PARTS, bool OUT>
 __global__ __launch_bounds__(TM_WAVE) void gla_scan_vec_kernel(const T* __restrict__ proj, int ld, int q_off, int k_off, int v_off,
                                                               const float* __restrict__ decay, float* __restrict__ o,
                                                               float* __restrict__ state, const int* __restrict__ cu_q_lens,
                                                               const int* __restrict__ state_slots, int H, int D, int Dv,
                                                               float q_scale) {
     constexpr int EV = Piece<T>::N, NQ = RMAX / EV, NA = RMAX / 4;
-    const int lane = threadIdx.x, part = lane % GLA_PARTS;
-    const int e = blockIdx.x * GLA_COLS + lane / GLA_PARTS;
+    const int lane = threadIdx.x, part = lane % PARTS;
+    const int e = blockIdx.x * (TM_WAVE / PARTS) + lane / PARTS;
     const int h = blockIdx.y, s = blockIdx.z;
-    const int R = D / GLA_PARTS;                      // a multiple of EV (and of 4): the host checks
+    const int R = D / PARTS;                          // a multiple of EV (and of 4): the host checks
     const int nq = R / EV, na = R / 4;
     const int d0 = part * R;
     const bool col = e < Dv;
@@ -112,7 +114,7 @@ __global__ __launch_bounds__(TM_WAVE) void gla_scan_vec_kernel(const T* __restri
 #pragma unroll
         for (int i = 0; i < NQ; ++i)
             if (i < nq) {
-                cq[i] = *(const uint4*)(row + head_q + i * EV);
+                if (OUT) cq[i] = *(const uint4*)(row + head_q + i * EV);
                 ck[i] = *(const uint4*)(row + head_k + i * EV);
             }
 #pragma unroll
@@ -128,7 +130,7 @@ __global__ __launch_bounds__(TM_WAVE) void gla_scan_vec_kernel(const T* __restri
 #pragma unroll
             for (int i = 0; i < NQ; ++i)
                 if (i < nq) {
-                    nq_[i] = *(const uint4*)(row + head_q + i * EV);
+                    if (OUT) nq_[i] = *(const uint4*)(row + head_q + i * EV);
                     nk_[i] = *(const uint4*)(row + head_k + i * EV);
                 }
 #pragma unroll
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(TM_WAVE) void gla_scan_vec_kernel(const T* __restri
         for (int i = 0; i < NQ; ++i) {
             if (i < nq) {
                 float qf[EV], kf[EV];
-                Piece<T>::unpack(cq[i], qf);
+                if (OUT) Piece<T>::unpack(cq[i], qf);
                 Piece<T>::unpack(ck[i], kf);
 #pragma unroll
                 for (int j = 0; j < EV; ++j) {
@@ -150,16 +152,19 @@ __global__ __launch_bounds__(TM_WAVE) void gla_scan_vec_kernel(const T* __restri
                     const float a = (r % 4 == 0) ? a4.x : (r % 4 == 1) ? a4.y : (r % 4 == 2) ? a4.z : a4.w;
                     const float kv = kf[j] * cv;
                     S[r] = a * S[r] + kv;
-                    acc += S[r] * (qf[j] * q_scale);
+                    if (OUT) acc += S[r] * (qf[j] * q_scale);
                 }
             }
         }
-        acc += __shfl_xor(acc, 1, TM_WAVE);
-        acc += __shfl_xor(acc, 2, TM_WAVE);
-        if (col && part == 0) o[((size_t)t * H + h) * Dv + e] = acc;
+        if (OUT) {
+            acc += __shfl_xor(acc, 1, TM_WAVE);
+            acc += __shfl_xor(acc, 2, TM_WAVE);
+            if (PARTS == 8) acc += __shfl_xor(acc, 4, TM_WAVE);
+            if (col && part == 0) o[((size_t)t * H + h) * Dv + e] = acc;
+        }
 #pragma unroll
         for (int i = 0; i < NQ; ++i) {
-            cq[i] = nq_[i];
+            if (OUT) cq[i] = nq_[i];
             ck[i] = nk_[i];
         }
 #pragma unroll
@@ -172,9 +177,9 @@ __global__ __launch_bounds__(TM_WAVE) void gla_scan_vec_kernel(const T* __restri
 }
 
 template <typename T>
-static bool gla_scan_in_pieces(const void* proj, int ld, int q_off, int k_off, const float* decay, int D) {
+static bool gla_scan_in_pieces(const void* proj, int ld, int q_off, int k_off, const float* decay, int D, int parts) {
     constexpr int EV = Piece<T>::N;
-    return D % (GLA_PARTS * EV) == 0 && ld % EV == 0 && q_off % EV == 0 && k_off % EV == 0 && ((uintptr_t)proj % 16) == 0 &&
+    return D % (parts * EV) == 0 && ld % EV == 0 && q_off % EV == 0 && k_off % EV == 0 && ((uintptr_t)proj % 16) == 0 &&
            ((uintptr_t)decay % 16) == 0;
 }
 
@@ -183,14 +188,24 @@ static int launch_gla_scan(const void* proj, int ld, int q_off, int k_off, int v
                            const int* cu, const int* slots, int S, int H, int D, int Dv, float q_scale, hipStream_t stream) {
     const dim3 grid((Dv + GLA_COLS - 1) / GLA_COLS, H, S);
     const int R = (D + GLA_PARTS - 1) / GLA_PARTS;
-    if (R <= 32 && gla_scan_in_pieces<T>(proj, ld, q_off, k_off, decay, D)) {       // beyond 32 rows a lane the registers do not hold two tokens
-#define GLA_VEC(RM) gla_scan_vec_kernel<T, RM><<<grid, TM_WAVE, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu, slots, H, D, Dv, q_scale)
-        if (R <= 16) GLA_VEC(16);
-        else GLA_VEC(32);
-#undef GLA_VEC
+    // o == nullptr: only the states are wanted (the first scan of a portion in segments)
+#define GLA_VEC(RM, P, OUT_)                                                                                                     \
+    gla_scan_vec_kernel<T, RM, P, OUT_><<<dim3((Dv + TM_WAVE / P - 1) / (TM_WAVE / P), H, S), TM_WAVE, 0, stream>>>(              \
+        (const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu, slots, H, D, Dv, q_scale)
+    if (D / 8 <= 32 && gla_scan_in_pieces<T>(proj, ld, q_off, k_off, decay, D, 8)) {           // eight lanes a column
+        if (D / 8 <= 16) { if (o) GLA_VEC(16, 8, true); else GLA_VEC(16, 8, false); }
+        else { if (o) GLA_VEC(32, 8, true); else GLA_VEC(32, 8, false); }
         TM_CHECK_LAUNCH();
         return TM_OK;
     }
+    if (R <= 32 && gla_scan_in_pieces<T>(proj, ld, q_off, k_off, decay, D, GLA_PARTS)) {       // beyond 32 rows a lane the registers do not hold two tokens
+        if (R <= 16) { if (o) GLA_VEC(16, 4, true); else GLA_VEC(16, 4, false); }
+        else { if (o) GLA_VEC(32, 4, true); else GLA_VEC(32, 4, false); }
+        TM_CHECK_LAUNCH();
+        return TM_OK;
+    }
+#undef GLA_VEC
+    if (!o) return TM_ERR_ARG;                                  // the scan without results exists for rows in 16-byte pieces only
     if (R <= 16)
         gla_scan_kernel<T, 16><<<grid, TM_WAVE, 0, stream>>>((const T*)proj, ld, q_off, k_off, v_off, decay, o, state, cu, slots, H,
                                                             D, Dv, q_scale);
@@ -204,6 +219,20 @@ static int launch_gla_scan(const void* proj, int ld, int q_off, int k_off, int v
     return TM_OK;
 }
 
+// Does the scan of these operands run in 16-byte pieces (and so also without results, o == nullptr)?
+template <typename T>
+static bool gla_scan_pieces_any(const void* proj, int ld, int q_off, int k_off, const float* decay, int D) {
+    return (D / 8 <= 32 && gla_scan_in_pieces<T>(proj, ld, q_off, k_off, decay, D, 8)) ||
+           ((D + GLA_PARTS - 1) / GLA_PARTS <= 32 && gla_scan_in_pieces<T>(proj, ld, q_off, k_off, decay, D, GLA_PARTS));
+}
+
+extern "C" int tm_gla_scan_in_pieces(int dtype, const void* proj, int ld, int q_off, int k_off, const float* decay, int D) {
+    if (D <= 0) return 0;
+    if (dtype == TM_F32) return gla_scan_pieces_any<float>(proj, ld, q_off, k_off, decay, D) ? 1 : 0;
+    if (dtype == TM_BF16) return gla_scan_pieces_any<bf16_t>(proj, ld, q_off, k_off, decay, D) ? 1 : 0;
+    return 0;
+}
+
 // proj rows hold q [H, D] at q_off, k [H, D] at k_off, v [H, Dv] at v_off (element offsets into a row of ld elements);
 // decay float32 [T, H, D]; o float32 [T, H, Dv]; state float32 [slots, H, D, Dv]; request s of the step owns rows
 // cu_q_lens[s] .. cu_q_lens[s + 1] - 1 and the state row state_slots[s].
@@ -211,7 +240,7 @@ extern "C" int tm_gla_scan(const void* proj, int ld, int q_off, int k_off, int v
                            float* state, const int* cu_q_lens, const int* state_slots, int S, int H, int D, int Dv,
                            float q_scale, hipStream_t stream) {
     if (S <= 0) return TM_OK;
-    if (H <= 0 || D <= 0 || D > 256 || Dv <= 0 || H > 65535 || S > 65535 || !proj || !decay || !o || !state || !cu_q_lens ||
+    if (H <= 0 || D <= 0 || D > 256 || Dv <= 0 || H > 65535 || S > 65535 || !proj || !decay || !state || !cu_q_lens ||
         !state_slots || q_off < 0 || k_off < 0 || v_off < 0 || ld < q_off + H * D || ld < k_off + H * D || ld < v_off + H * Dv)
         return TM_ERR_ARG;
     if (dtype == TM_F32) return launch_gla_scan<float>(proj, ld, q_off, k_off, v_off, decay, o, state, cu_q_lens, state_slots, S, H, D, Dv, q_scale, stream);

@@ -1153,10 +1153,16 @@ def gla_decay(z: torch.Tensor, tau: float, out: torch.Tensor | None = None) -> t
     return out
 
 
-def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torch.Tensor, o: torch.Tensor, state: torch.Tensor,
+def gla_scan_states_only(proj: torch.Tensor, q_off: int, k_off: int, decay: torch.Tensor, D: int) -> bool:
+    """Can ``gla_scan`` run these operands without results (``o`` None), advancing the states only?"""
+    ld = proj.stride(0) if proj.shape[0] > 1 else max(proj.shape[1], proj.stride(0))
+    return bool(library().tm_gla_scan_in_pieces(c_int(code(proj.dtype)), _p(proj), c_int(ld), c_int(q_off), c_int(k_off), _p(decay), c_int(D)))
+
+
+def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torch.Tensor, o: torch.Tensor | None, state: torch.Tensor,
              cu_q_lens: torch.Tensor, state_slots: torch.Tensor, num_seqs: int, H: int, D: int, Dv: int, q_scale: float) -> torch.Tensor:
     """The recurrence S = diag(decay_t) S + k_t v_t^T, o_t = S^T (q_scale * q_t) over the rows of each request of the
-    step in order, from and to the request's state row. proj [T, ld] holds q, k [H*D] and v [H*Dv] at the given column
+    step in order, from and to the request's state row (``o`` None where ``gla_scan_states_only``: the states alone). proj [T, ld] holds q, k [H*D] and v [H*Dv] at the given column
     offsets; decay float32 [T, H*D]; o float32 [T, H*Dv]; state float32 [slots, H, D, Dv]; cu_q_lens int32 [S+1];
     state_slots int32 [S]."""
     _gpu(proj, decay, o, state, cu_q_lens, state_slots)
@@ -1166,7 +1172,10 @@ def gla_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torc
     for off, n in ((q_off, H * D), (k_off, H * D), (v_off, H * Dv)):
         _need(0 <= off and off + n <= ld_cols, "gla_scan: q, k, v lie inside a row of proj")
     _need(decay.dtype == torch.float32 and decay.is_contiguous() and tuple(decay.shape) == (T, H * D), f"gla_scan: decay float32 [{T}, {H * D}]")
-    _need(o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (T, H * Dv), f"gla_scan: o float32 [{T}, {H * Dv}]")
+    if o is not None:
+        _need(o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (T, H * Dv), f"gla_scan: o float32 [{T}, {H * Dv}]")
+    else:
+        _need(gla_scan_states_only(proj, q_off, k_off, decay, D), "gla_scan: these operands are not scanned without results")
     _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, D, Dv),
           f"gla_scan: state float32 [slots, {H}, {D}, {Dv}]")
     _ints(cu_q_lens, num_seqs + 1, "cu_q_lens")

@@ -140,7 +140,8 @@ class GatedLinearAttention(Mixer):
             return
         cu_seg, ids, first, n_seg = self._segments(step, proj.device)
         local = torch.zeros((n_seg, H, D, Dv), dtype=torch.float32, device=proj.device)
-        ops.gla_scan(proj, 0, ks, 2 * ks, decay, o, local, cu_seg, ids, n_seg, H, D, Dv, scale)         # o: overwritten below
+        states_only = ops.gla_scan_states_only(proj, 0, ks, decay, D)                                    # else o is written and overwritten below
+        ops.gla_scan(proj, 0, ks, 2 * ks, decay, None if states_only else o, local, cu_seg, ids, n_seg, H, D, Dv, scale)
         products = torch.empty((n_seg, ks), dtype=torch.float32, device=proj.device)
         ops.gla_segment_decay(decay, cu_seg, n_seg, products)
         start = torch.empty_like(local)
