@@ -147,7 +147,7 @@ def _run_cuts(attn, pools, manager, runner, x, dt, cuts):
 
 @pytest.mark.parametrize("dt", DTS)
 @pytest.mark.parametrize("H,G,D,Dv,rot,chunk", [(6, 2, 24, 16, 12, 24), (4, 4, 32, 40, 32, 50), (5, 1, 20, 68, 0, None),
-                                                 (2, 1, 128, 128, 64, 100), (3, 3, 6, 2, 2, 1), (8, 1, 48, 64, 48, 40),
+                                                 (2, 1, 128, 128, 64, 100), (3, 3, 6, 2, 2, 1), (8, 2, 40, 56, 24, 40),
                                                  (3, 1, 104, 100, 8, None)])
 @pytest.mark.parametrize("page", [8, 16, 64])           # pages of 16 and more: prompt portions of bfloat16 run on the matrix unit
 def test_sigmoid_attention_whole_then_portions_then_tokens(dt, H, G, D, Dv, rot, chunk, page):
