@@ -36,7 +36,7 @@ def close(got, want, dt, what, bf16=2.0 ** -7):
 # ----------------------------------------------------------------------------------------------- mechanisms alone
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("hidden,groups", [(96, 3), (96, 1), (200, 8), (1024, 2), (60, 5)])
+@pytest.mark.parametrize("hidden,groups", [(96, 3), (96, 1), (200, 8), (1024, 2), (60, 5), (256, 8), (256, 16), (4096, 4), (5120, 2)])
 def test_norm_in_groups_around_a_sublayer(dt, hidden, groups):
     from tokenmill_amd.parts import GroupRMSNorm, NormedInput, as_tensor
     torch.manual_seed(hidden + groups)
