@@ -504,18 +504,20 @@ def test_greedy_generation_through_the_engine_and_its_graphs(models):
     prompts = [random_ids(n, 211, 500 + i) for i, n in enumerate([12, 3, 30, 7, 21, 16, 45, 25, 5, 18])]
     params = [SamplingParams(max_tokens=8 + 5 * (i % 4), ignore_eos=True) for i in range(len(prompts))]
     outs = {}
-    for mode in ("eager", "graphs", "chunked"):
+    for mode in ("eager", "graphs", "chunked", "ahead"):
         eng = LLMEngine(EngineConfig(model=str(d), dtype="float32", block_size=8, num_blocks=48, max_model_len=96,
                                      max_num_seqs=4, max_num_batched_tokens=32 if mode == "chunked" else 64, watermark=0.0,
-                                     hip_graphs=mode != "eager", enable_chunked_prefill=mode == "chunked"))
+                                     hip_graphs=mode != "eager", enable_chunked_prefill=mode == "chunked",
+                                     pipeline_decode=mode == "ahead"))
         kinds = [type(p).__name__ for p in eng.runner.program.foreign_parts]
         assert kinds.count("GatedLinearAttention") == 2 and kinds.count("SigmoidAttention") == 2
         outs[mode] = eng.generate(prompts, params)
-        if mode == "graphs":
+        if mode in ("graphs", "ahead"):
             assert eng.runner.graphs.stateful_ok and eng.runner.graphs.replays > 10
+        assert (eng.stats["steps_ahead"] > 5) == (mode == "ahead")      # decode steps queued behind the running one advance each state once
         assert eng.cache.num_free_pages == eng.cache.num_pages
     tokens = {m: [list(o) for o in outs[m]] for m in outs}
-    assert tokens["eager"] == tokens["graphs"] == tokens["chunked"]
+    assert tokens["eager"] == tokens["graphs"] == tokens["chunked"] == tokens["ahead"]
     exempt = 0
     for prompt, toks in zip(prompts, tokens["eager"]):
         rows = M.logits(w, cfg, prompt + toks[:-1], torch.float32)[len(prompt) - 1:]
