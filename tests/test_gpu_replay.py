@@ -79,7 +79,8 @@ def poison_freed_pages(session):
             if pages:
                 idx = torch.tensor(pages, dtype=torch.long, device=pools.k[g].device)
                 pools.k[g].index_fill_(1, idx, math.nan)
-                pools.v[g].index_fill_(1, idx, math.nan)
+                if pools.v[g] is not None:            # a group whose values are part of its key rows has no value pool
+                    pools.v[g].index_fill_(1, idx, math.nan)
             return plain_release(pages)
 
         alloc.release = release

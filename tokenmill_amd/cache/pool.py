@@ -11,7 +11,7 @@ from __future__ import annotations
 
 import torch
 
-from tokenmill_amd.parts.base import KVCacheSpec, KVCacheView, StateSpec, StateView
+from tokenmill_amd.parts.base import KVCacheSpec, KVCacheView, LayerCacheSpec, StateSpec, StateView
 
 
 def group_specs(cache_specs: list) -> tuple[list[KVCacheSpec], list[int | None]]:
@@ -19,6 +19,8 @@ def group_specs(cache_specs: list) -> tuple[list[KVCacheSpec], list[int | None]]
     groups: list[KVCacheSpec] = []
     of_call: list[int | None] = []
     for spec in cache_specs:
+        if isinstance(spec, LayerCacheSpec):
+            spec = spec.kv
         if isinstance(spec, KVCacheSpec):
             if spec not in groups:
                 groups.append(spec)
@@ -41,21 +43,27 @@ class CachePools:
         self.k = [torch.zeros((len(members[g]), counts[g], page_size, s.kv_heads, s.head_dim), dtype=dtype,
                               device=device) for g, s in enumerate(self.groups)]
         self.v = [torch.zeros((len(members[g]), counts[g], s.kv_heads, s.value_dim, page_size), dtype=dtype,
-                              device=device) for g, s in enumerate(self.groups)]
+                              device=device) if s.values else None for g, s in enumerate(self.groups)]
         self.states: dict[int, torch.Tensor] = {}
         views: list = [None] * len(specs)
         for g, calls in enumerate(members):
             for idx, j in enumerate(calls):
-                views[j] = KVCacheView(self.k[g][idx], self.v[g][idx], g, True)
+                views[j] = KVCacheView(self.k[g][idx], self.v[g][idx] if self.v[g] is not None else None, g, True)
         for j, spec in enumerate(specs):
+            beside = isinstance(spec, LayerCacheSpec)
+            if beside:
+                spec = spec.state
             if isinstance(spec, StateSpec):
                 # one row more than there are slots: where the padding rows of a replayed step put their state
-                self.states[j] = torch.zeros((num_state_slots + 1, *spec.shape), dtype=spec.dtype, device=device)
-                views[j] = StateView(self.states[j])
+                self.states[j] = torch.zeros((num_state_slots + 1, *spec.shape), dtype=spec.dtype or dtype, device=device)
+                if beside and views[j] is not None:
+                    views[j].state = self.states[j]
+                else:
+                    views[j] = StateView(self.states[j])
         for j, call in enumerate(model.run):
             if call.cache_of is not None:
                 src = views[call.cache_of]
-                views[j] = KVCacheView(src.k, src.v, src.group, False) if isinstance(src, KVCacheView) else src
+                views[j] = KVCacheView(src.k, src.v, src.group, False, src.state) if isinstance(src, KVCacheView) else src
         self.views = views
 
     @property
@@ -78,11 +86,12 @@ class CachePools:
 
     @property
     def nbytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.k + self.v) + \
+        return sum(t.numel() * t.element_size() for t in self.k + self.v if t is not None) + \
             sum(t.numel() * t.element_size() for t in self.states.values())
 
     @staticmethod
     def bytes_per_token(model, dtype) -> int:
         """Cache bytes one token takes over all layers (reference src/infer/config.py:37-39)."""
         size = torch.empty((), dtype=dtype).element_size()
-        return sum(s.kv_heads * (s.head_dim + s.value_dim) * size for s in model.cache_specs() if isinstance(s, KVCacheSpec))
+        specs = [s.kv if isinstance(s, LayerCacheSpec) else s for s in model.cache_specs()]
+        return sum(s.kv_heads * (s.head_dim + s.value_dim) * size for s in specs if isinstance(s, KVCacheSpec))

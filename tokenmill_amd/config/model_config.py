@@ -236,6 +236,111 @@ class ModinexConfig:
                 raise ConfigError(f"layers[{i}]: ff must be positive")
 
 
+@dataclass(frozen=True)
+class LusolixLayer:
+    """One entry of a Lusolix model's list of layers."""
+    type: str                                  # "latent_attention"
+    mixer: dict                                # the mixer's sizes and constants, as config.json gives them
+    mlp: dict | None                           # {"kind": "dense", "ff": F} | {"kind": "moe", "ff": F, "experts": E, "top": k} | None
+
+
+@dataclass(frozen=True)
+class LusolixConfig:
+    """The Lusolix decoder: token embedding plus a learned position table; pre-norm layers (layer norm with bias) whose
+    sublayers' results are scaled by ``residual_mult`` and gated on their way into the residual stream; a short causal
+    convolution of ``canon.taps`` taps in front of every mixer; attention through a shared latent inside a sliding
+    window; a dense feed-forward with the PolyNorm activation or experts chosen by a table of the token id; the output
+    head is the embedding table. Every size and constant that can differ between two models is read from config.json."""
+
+    vocab_size: int
+    hidden_size: int
+    max_position_embeddings: int
+    norm_eps: float
+    residual_mult: float
+    conv_taps: int
+    layers: tuple[LusolixLayer, ...]
+    eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
+
+    architecture = "Lusolix"
+    MIXERS = ("latent_attention",)
+    MLPS = ("dense", "moe")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, raw: dict, generation: dict | None = None) -> "LusolixConfig":
+        norm = _require(raw, "norm")
+        layers = []
+        for i, entry in enumerate(_require(raw, "layers")):
+            kind = entry.get("type")
+            if kind not in cls.MIXERS:
+                raise ConfigError(f"layers[{i}]: type '{kind}' is not one of {list(cls.MIXERS)}")
+            mixer = entry.get("mixer")
+            if not isinstance(mixer, dict):
+                raise ConfigError(f"layers[{i}] has no 'mixer' sizes")
+            for key in ("heads", "dim", "rot_dim", "vdim", "q_rank", "kv_rank", "scale"):
+                if mixer.get(key) is None:
+                    raise ConfigError(f"layers[{i}]: the {kind} mixer has no '{key}'")
+            mlp = entry.get("mlp")
+            if mlp is not None:
+                how = mlp.get("kind", "dense")
+                if how not in cls.MLPS:
+                    raise ConfigError(f"layers[{i}]: feed-forward kind '{how}' is not one of {list(cls.MLPS)}")
+                if how == "dense":
+                    if mlp.get("ff") is None:
+                        raise ConfigError(f"layers[{i}]: the feed-forward has no 'ff' width")
+                    mlp = {"kind": "dense", "ff": int(mlp["ff"])}
+                else:
+                    expert, router = mlp.get("expert") or {}, mlp.get("router") or {}
+                    for where, key in ((expert, "ff"), (router, "experts"), (router, "top")):
+                        if where.get(key) is None:
+                            raise ConfigError(f"layers[{i}]: the experts have no '{key}'")
+                    mlp = {"kind": "moe", "ff": int(expert["ff"]), "experts": int(router["experts"]), "top": int(router["top"])}
+            layers.append(LusolixLayer(kind, dict(mixer), mlp))
+        cfg = cls(vocab_size=int(_require(raw, "vocab")), hidden_size=int(_require(raw, "width")),
+                  max_position_embeddings=int(_require(raw, "max_positions")), norm_eps=float(_require(norm, "eps")),
+                  residual_mult=float(raw.get("residual_mult", 1.0)), conv_taps=int((raw.get("canon") or {}).get("taps", 0)),
+                  layers=tuple(layers), eos_token_ids=collect_eos_ids(([generation] if generation else []) + [raw]))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        for name in ("vocab_size", "hidden_size", "max_position_embeddings"):
+            if getattr(self, name) <= 0:
+                raise ConfigError(f"{name} must be positive, got {getattr(self, name)}")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if not 0 <= self.conv_taps <= 16:
+            raise ConfigError(f"canon.taps {self.conv_taps}: 0 (none) to 16")
+        if not self.layers:
+            raise ConfigError("a model needs at least one layer")
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            for key in ("heads", "dim", "vdim", "q_rank", "kv_rank"):
+                if int(m[key]) <= 0:
+                    raise ConfigError(f"layers[{i}]: {key} must be positive")
+            if int(m["rot_dim"]) < 0:
+                raise ConfigError(f"layers[{i}]: rot_dim must not be negative")
+            rot = m.get("rot")
+            if rot:
+                dims = int(rot.get("dims", 0))
+                if dims < 0 or dims % 2 or dims > int(m["rot_dim"]):
+                    raise ConfigError(f"layers[{i}]: rot.dims {dims} must be even and at most rot_dim {m['rot_dim']}")
+                if dims and not float(rot.get("base", 0)) > 0:
+                    raise ConfigError(f"layers[{i}]: rot.base must be positive")
+            mask = m.get("mask")
+            if mask and mask.get("size") is not None and int(mask["size"]) <= 0:
+                raise ConfigError(f"layers[{i}]: mask.size must be positive")
+            mlp = layer.mlp
+            if mlp is not None:
+                if mlp["ff"] <= 0:
+                    raise ConfigError(f"layers[{i}]: ff must be positive")
+                if mlp["kind"] == "moe" and not 0 < mlp["top"] <= mlp["experts"]:
+                    raise ConfigError(f"layers[{i}]: {mlp['top']} of {mlp['experts']} experts")
+
+
 def read_json(path: Path) -> dict:
     try:
         return json.loads(path.read_text())

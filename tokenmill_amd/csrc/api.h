@@ -167,6 +167,43 @@ int tm_gla_segment_decay(const float* decay, const int* cu_seg, float* P, int n_
 int tm_gla_combine(float* state, const int* state_slots, const int* first_seg, const float* P, const float* local,
                    float* start, int S, int HD, int Dv, hipStream_t stream);
 
+// Layer norm with weight and bias behind a gated, scaled residual add (layer_norm.hip):
+// v = resid[r] + mult * y[r] * sigmoid(gate[r]) (gate null: no gate; y null: nothing added), written back to resid when
+// every row runs (rows null); out[r] = layer_norm(v) * w + b (out null: the add alone). y, gate, out of type `dtype`.
+int tm_layer_norm(float* resid, const void* y, const void* gate, float mult, const int* rows, const float* w, const float* b,
+                  void* out, int dtype, int R, int hidden, float eps, hipStream_t stream);
+// out[t] = h[t] + sum_j w[:, j] * h[t - taps + 1 + j] over a request's rows, the rows before the step's first from the
+// request's state [taps - 1, width] (row state_slots[s] of `state`); then tm_short_conv_state makes the state the last
+// taps - 1 rows the request has seen. h, out, w [width, taps] and state of type `dtype`; taps up to 16.
+int tm_short_conv(const void* h, void* out, const void* w, const void* state, const int* cu_q_lens, const int* state_slots,
+                  const int* seq_of_token, int T, int width, int taps, int dtype, hipStream_t stream);
+int tm_short_conv_state(const void* h, void* state, const int* cu_q_lens, const int* state_slots, int S, int width, int taps,
+                        int dtype, hipStream_t stream);
+// out = a N(z) + b N(z^2) + c N(z^3) + e with coef = (a, b, c, e) on the device, N(v) = v / sqrt(mean(v^2) + eps) per row.
+int tm_poly_norm(const float* z, const float* coef, void* out, int dtype, int T, int F, float eps, hipStream_t stream);
+
+// Attention over a shared latent (latent.hip): see the head of that file.
+int tm_latent_prepare(const float* low, int ld, int Lq, int Lk, int Dr, int rot, const float* wq, const float* wk, float eps,
+                      const float* cos_t, const float* sin_t, const int* positions, const int* slots, void* cq, void* pool,
+                      int dtype, int T, hipStream_t stream);
+int tm_heads_matmul(const void* A, int lda, int a_head, const void* B, void* C, int ldc, int c_head, const float* gate, int ldg,
+                    int T, int H, int K, int N, int dtype, hipStream_t stream);
+int tm_rotate_heads(const void* src, int ld_src, int src_head, void* dst, int ld_dst, int dst_head, int T, int H, int Dr, int rot,
+                    const float* cos_t, const float* sin_t, const int* positions, int dtype, hipStream_t stream);
+int tm_attn_latent(const void* qa, int q_stride, void* out, int out_stride, const void* pool, const int* block_tables,
+                   int table_width, const int* seq_of_token, const int* positions, int T, int H, int Lk, int Dk, int page,
+                   float scale, int window, int dtype, hipStream_t stream);
+
+// Experts chosen by a table row of the token id (moe.hip): see the head of that file.
+int tm_moe_route(const int* ids, const int* table, int T, int top, int E, int tile_rows, int* slot_pair, int* pair_slot,
+                 int* tiles, int* n_tiles, hipStream_t stream);
+int tm_moe_gate_up(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
+                   const int* n_tiles, int max_tiles, int K, int F, int dtype, hipStream_t stream);
+int tm_moe_down(const void* act, const void* W, float* part, const int* tiles, const int* n_tiles, int max_tiles, int F, int N,
+                int dtype, hipStream_t stream);
+int tm_moe_combine(const float* part, const int* pair_slot, void* y, int T, int top, float weight, int N, int dtype,
+                   hipStream_t stream);
+
 int tm_argmax_work_chunks(int V);
 int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);
 

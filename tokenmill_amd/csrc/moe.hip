@@ -1,0 +1,196 @@
+// A feed-forward of many small experts of which every token uses a few, chosen by a table row of its token id.
+//
+//   pair p = (token t = p / top, choice k = p % top) goes to expert e(p) = table[id[t] * top + k]
+//   tm_moe_route     sorts the pairs by expert: slot_pair[slot] = p, pair_slot[p] = slot, and cuts every expert's run of
+//                    slots into tiles of `tile_rows` rows: tiles[i] = (expert, first slot, rows), n_tiles[0] = their number
+//   tm_moe_gate_up   act[slot] = silu(x[t] . Wg[e]^T) * (x[t] . Wu[e]^T)          W [E, 2F, K]: gate rows, then up rows
+//   tm_moe_down      part[slot] = act[slot] . Wd[e]^T  (32-bit)                    Wd [E, N, F]
+//   tm_moe_combine   y[t] = sum_k weight * part[pair_slot[t * top + k]], k ascending, rounded once
+//
+// All of it runs from device data (no count crosses to the host), so a step can be recorded into a graph. Which slot a
+// pair gets inside its expert's run may differ from run to run (the cursor is an atomic counter); a row's result does not
+// depend on its slot: every element is summed over k in ascending order by one thread.
+#include "common.h"
+#include "api.h"
+
+#define MR_THREADS 1024
+#define MOE_MAX_EXPERTS 1024
+
+__global__ __launch_bounds__(MR_THREADS) void moe_route_kernel(const int* __restrict__ ids, const int* __restrict__ table, int T,
+                                                               int top, int E, int tile_rows, int* __restrict__ slot_pair,
+                                                               int* __restrict__ pair_slot, int* __restrict__ tiles,
+                                                               int* __restrict__ n_tiles) {
+    __shared__ int cnt[MOE_MAX_EXPERTS];
+    __shared__ int off[MOE_MAX_EXPERTS + 1];
+    const int P = T * top;
+    for (int e = threadIdx.x; e < E; e += MR_THREADS) cnt[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < P; p += MR_THREADS) {
+        const int e = table[(size_t)ids[p / top] * top + p % top];
+        atomicAdd(&cnt[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, n = 0;
+        for (int e = 0; e < E; ++e) {
+            off[e] = at;
+            for (int r = 0; r < cnt[e]; r += tile_rows) {
+                tiles[3 * n] = e;
+                tiles[3 * n + 1] = at + r;
+                tiles[3 * n + 2] = min(tile_rows, cnt[e] - r);
+                ++n;
+            }
+            at += cnt[e];
+            cnt[e] = 0;
+        }
+        off[E] = at;
+        n_tiles[0] = n;
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < P; p += MR_THREADS) {
+        const int e = table[(size_t)ids[p / top] * top + p % top];
+        const int slot = off[e] + atomicAdd(&cnt[e], 1);
+        slot_pair[slot] = p;
+        pair_slot[p] = slot;
+    }
+}
+
+extern "C" int tm_moe_route(const int* ids, const int* table, int T, int top, int E, int tile_rows, int* slot_pair, int* pair_slot,
+                            int* tiles, int* n_tiles, hipStream_t stream) {
+    if (!ids || !table || !slot_pair || !pair_slot || !tiles || !n_tiles || T < 0 || top <= 0 || E <= 0 || E > MOE_MAX_EXPERTS ||
+        tile_rows <= 0 || (long long)T * top > 0x3fffffffLL)
+        return TM_ERR_ARG;
+    moe_route_kernel<<<1, MR_THREADS, 0, stream>>>(ids, table, T, top, E, tile_rows, slot_pair, pair_slot, tiles, n_tiles);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ grouped products
+
+#define MG_TM 32            // rows of a tile (tile_rows of the route)
+#define MG_TN 64
+#define MG_TK 16
+
+// GATED: C[slot, n] = silu(a . W[e][n]) * (a . W[e][F + n]), a = A[slot_pair[slot] / top]; C of type T.
+// else : C[slot, n] = A[slot] . W[e][n]; C float32.
+template <typename T, bool GATED>
+__global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ A, int lda, const int* __restrict__ slot_pair, int top,
+                                                          const T* __restrict__ W, void* __restrict__ Cv, int ldc,
+                                                          const int* __restrict__ tiles, const int* __restrict__ n_tiles, int K,
+                                                          int N) {
+    if ((int)blockIdx.x >= n_tiles[0]) return;
+    __shared__ float As[MG_TM][MG_TK + 1];
+    __shared__ float Bs[GATED ? 2 : 1][MG_TK][MG_TN + 1];
+    __shared__ int src[MG_TM];
+    const int e = tiles[3 * blockIdx.x], slot0 = tiles[3 * blockIdx.x + 1], rows = tiles[3 * blockIdx.x + 2];
+    const int n0 = blockIdx.y * MG_TN;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const T* We = W + (size_t)e * (GATED ? 2 : 1) * N * K;
+    if (threadIdx.x < MG_TM)
+        src[threadIdx.x] = threadIdx.x < rows ? (GATED ? slot_pair[slot0 + threadIdx.x] / top : slot0 + (int)threadIdx.x) : -1;
+    __syncthreads();
+    float acc[2][4] = {}, acu[2][4] = {};
+    for (int k0 = 0; k0 < K; k0 += MG_TK) {
+        for (int i = threadIdx.x; i < MG_TM * MG_TK; i += 256) {
+            const int r = i / MG_TK, k = i % MG_TK;
+            As[r][k] = (src[r] >= 0 && k0 + k < K) ? Elem<T>::load(A + (size_t)src[r] * lda + k0 + k) : 0.f;
+        }
+        for (int i = threadIdx.x; i < MG_TK * MG_TN; i += 256) {
+            const int n = i / MG_TK, k = i % MG_TK;
+            const bool in = n0 + n < N && k0 + k < K;
+            Bs[0][k][n] = in ? Elem<T>::load(We + (size_t)(n0 + n) * K + k0 + k) : 0.f;
+            if (GATED) Bs[1][k][n] = in ? Elem<T>::load(We + (size_t)(N + n0 + n) * K + k0 + k) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < MG_TK; ++k) {
+            const float a0 = As[ty * 2][k], a1 = As[ty * 2 + 1][k];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float b = Bs[0][k][tx * 4 + j];
+                acc[0][j] += a0 * b;
+                acc[1][j] += a1 * b;
+                if (GATED) {
+                    const float u = Bs[1][k][tx * 4 + j];
+                    acu[0][j] += a0 * u;
+                    acu[1][j] += a1 * u;
+                }
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int r = ty * 2 + i;
+        if (r >= rows) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            if (GATED) {
+                const float g = acc[i][j], u = acu[i][j];
+                Elem<T>::store((T*)Cv + (size_t)(slot0 + r) * ldc + n, g / (1.0f + __expf(-g)) * u);
+            } else {
+                ((float*)Cv)[(size_t)(slot0 + r) * ldc + n] = acc[i][j];
+            }
+        }
+    }
+}
+
+extern "C" int tm_moe_gate_up(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
+                              const int* n_tiles, int max_tiles, int K, int F, int dtype, hipStream_t stream) {
+    if (!x || !slot_pair || !W || !act || !tiles || !n_tiles || top <= 0 || K <= 0 || F <= 0 || ldx < K || max_tiles < 0) return TM_ERR_ARG;
+    if (dtype != TM_F32 && dtype != TM_BF16) return TM_ERR_ARG;
+    if (max_tiles == 0) return TM_OK;
+    dim3 grid(max_tiles, (F + MG_TN - 1) / MG_TN);
+    if (grid.y > 65535) return TM_ERR_ARG;
+    if (dtype == TM_F32)
+        moe_product_kernel<float, true><<<grid, 256, 0, stream>>>((const float*)x, ldx, slot_pair, top, (const float*)W, act, F, tiles,
+                                                                  n_tiles, K, F);
+    else
+        moe_product_kernel<bf16_t, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, slot_pair, top, (const bf16_t*)W, act, F, tiles,
+                                                                   n_tiles, K, F);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+extern "C" int tm_moe_down(const void* act, const void* W, float* part, const int* tiles, const int* n_tiles, int max_tiles, int F,
+                           int N, int dtype, hipStream_t stream) {
+    if (!act || !W || !part || !tiles || !n_tiles || F <= 0 || N <= 0 || max_tiles < 0) return TM_ERR_ARG;
+    if (dtype != TM_F32 && dtype != TM_BF16) return TM_ERR_ARG;
+    if (max_tiles == 0) return TM_OK;
+    dim3 grid(max_tiles, (N + MG_TN - 1) / MG_TN);
+    if (grid.y > 65535) return TM_ERR_ARG;
+    if (dtype == TM_F32)
+        moe_product_kernel<float, false><<<grid, 256, 0, stream>>>((const float*)act, F, nullptr, 1, (const float*)W, part, N, tiles,
+                                                                   n_tiles, F, N);
+    else
+        moe_product_kernel<bf16_t, false><<<grid, 256, 0, stream>>>((const bf16_t*)act, F, nullptr, 1, (const bf16_t*)W, part, N, tiles,
+                                                                    n_tiles, F, N);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ part, const int* __restrict__ pair_slot,
+                                                          T* __restrict__ y, int top, float weight, int N) {
+    const int t = blockIdx.x;
+    for (int c = threadIdx.x; c < N; c += 256) {
+        float s = 0.f;
+        for (int k = 0; k < top; ++k) s += weight * part[(size_t)pair_slot[t * top + k] * N + c];
+        Elem<T>::store(y + (size_t)t * N + c, s);
+    }
+}
+
+extern "C" int tm_moe_combine(const float* part, const int* pair_slot, void* y, int T, int top, float weight, int N, int dtype,
+                              hipStream_t stream) {
+    if (!part || !pair_slot || !y || T < 0 || top <= 0 || N <= 0) return TM_ERR_ARG;
+    if (dtype != TM_F32 && dtype != TM_BF16) return TM_ERR_ARG;
+    if (T == 0) return TM_OK;
+    if (dtype == TM_F32)
+        moe_combine_kernel<float><<<T, 256, 0, stream>>>(part, pair_slot, (float*)y, top, weight, N);
+    else
+        moe_combine_kernel<bf16_t><<<T, 256, 0, stream>>>(part, pair_slot, (bf16_t*)y, top, weight, N);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}

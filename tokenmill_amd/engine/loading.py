@@ -65,7 +65,10 @@ def load_random_model(config: dict, seed: int, dtype: torch.dtype, device: torch
     tensors = {}
     for name, spec in sorted(model.tensor_specs().items()):
         shape = spec.drawn_shape()
-        if spec.kind == "int":
+        if spec.kind == "int" and spec.init.startswith("distinct_below:"):
+            from tokenmill_amd.weights.random_init import distinct_rows
+            t = distinct_rows(shape, int(spec.init.split(":")[1]), g, device)
+        elif spec.kind == "int":
             t = torch.arange(int(torch.tensor(shape).prod()), dtype=torch.int32, device=device).reshape(shape)
         elif spec.init == "ones":
             t = torch.ones(shape, dtype=torch.float32, device=device)

@@ -1283,3 +1283,256 @@ def gla_combine(state: torch.Tensor, state_slots: torch.Tensor, first_seg: torch
     _need(num_seqs <= 65535, "gla_combine: at most 65,535 requests a step")
     _check(library().tm_gla_combine(_p(state), _p(state_slots), _p(first_seg), _p(seg_decay), _p(local), _p(start), c_int(num_seqs),
                                     c_int(H * D), c_int(Dv), _stream()), "gla_combine")
+
+
+# -------------------------------------------------------------------------------------------- layer norm, short convolution, PolyNorm
+
+def layer_norm(resid: torch.Tensor, y: torch.Tensor | None, gate: torch.Tensor | None, mult: float, w: torch.Tensor | None,
+               b: torch.Tensor | None, out: torch.Tensor | None, eps: float, rows: torch.Tensor | None = None, dtype=None):
+    """v = resid + mult * y * sigmoid(gate) (gate None: no gate; y None: nothing is added); with ``rows`` None every row runs
+    and v is written back to resid (float32 [T, hidden]); out = (v - mean) / sqrt(var + eps) * w + b (out None: the add
+    alone). With ``rows`` (int32 [R]) only those rows are read, resid stays as it is and out is [R, hidden]. y, gate and out
+    share one type; w, b are float32 [hidden]."""
+    _gpu(resid, y, gate, w, b, out, rows)
+    T, hidden = resid.shape
+    R = T if rows is None else rows.numel()
+    _need(resid.dtype == torch.float32 and resid.is_contiguous(), "layer_norm: the residual stream is contiguous float32")
+    _need(hidden <= 16384, "layer_norm: rows of up to 16,384 elements")
+    dt = dtype
+    for t, name in ((y, "y"), (gate, "gate")):
+        if t is not None:
+            _need(tuple(t.shape) == (T, hidden) and t.is_contiguous(), f"layer_norm: {name} must be contiguous [{T}, {hidden}]")
+            _need(dt in (None, t.dtype), "layer_norm: y, gate and out share one type")
+            dt = t.dtype
+    if out is not None:
+        _need(tuple(out.shape) == (R, hidden) and out.is_contiguous(), f"layer_norm: out must be contiguous [{R}, {hidden}]")
+        _need(dt in (None, out.dtype), "layer_norm: y, gate and out share one type")
+        dt = out.dtype
+        for t in (w, b):
+            _need(t is not None and t.dtype == torch.float32 and tuple(t.shape) == (hidden,) and t.is_contiguous(),
+                  f"layer_norm: weight and bias are float32 [{hidden}]")
+    _need(gate is None or y is not None, "layer_norm: a gate needs something to gate")
+    _need(dt is not None, "layer_norm: nothing to do")
+    if rows is not None:
+        _ints(rows, R, "rows")
+    _need(eps > 0, "layer_norm: eps must be positive")
+    _check(library().tm_layer_norm(_p(resid), _p(y), _p(gate), c_float(mult), _p(rows), _p(w), _p(b), _p(out), c_int(code(dt)),
+                                   c_int(R), c_int(hidden), c_float(eps), _stream()), "layer_norm")
+    return out
+
+
+def short_conv(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor | None, cu_q_lens: torch.Tensor, state_slots: torch.Tensor,
+               seq_of_token: torch.Tensor, num_seqs: int, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = h[t] + sum_j w[:, j] * h[t - taps + 1 + j] within each request (rows cu_q_lens[s] .. cu_q_lens[s + 1] - 1 of h),
+    the rows before the step's first taken from state[state_slots[s]] ([taps - 1, width]); afterwards that state holds the
+    last taps - 1 rows the request has seen. h, w [width, taps], state [slots, taps - 1, width] and out share one type."""
+    _gpu(h, w, state, cu_q_lens, state_slots, seq_of_token, out)
+    T, width = h.shape
+    taps = w.shape[1]
+    _need(h.is_contiguous() and out.is_contiguous() and out.shape == h.shape and out.dtype == h.dtype and out.data_ptr() != h.data_ptr(),
+          "short_conv: h and out are two contiguous tensors of one shape and type")
+    _need(tuple(w.shape) == (width, taps) and w.is_contiguous() and w.dtype == h.dtype and 1 <= taps <= 16,
+          "short_conv: w must be [width, taps] of h's type, taps up to 16")
+    if taps > 1:
+        _need(state is not None and state.dim() == 3 and tuple(state.shape[1:]) == (taps - 1, width) and state.is_contiguous()
+              and state.dtype == h.dtype, f"short_conv: state must be [slots, {taps - 1}, {width}] of h's type")
+    _ints(cu_q_lens, num_seqs + 1, "cu_q_lens")
+    _ints(state_slots, num_seqs, "state_slots")
+    _ints(seq_of_token, T, "seq_of_token")
+    lib = library()
+    _check(lib.tm_short_conv(_p(h), _p(out), _p(w), _p(state), _p(cu_q_lens), _p(state_slots), _p(seq_of_token), c_int(T),
+                             c_int(width), c_int(taps), c_int(code(h.dtype)), _stream()), "short_conv")
+    if taps > 1:
+        _check(lib.tm_short_conv_state(_p(h), _p(state), _p(cu_q_lens), _p(state_slots), c_int(num_seqs), c_int(width), c_int(taps),
+                                       c_int(code(h.dtype)), _stream()), "short_conv_state")
+    return out
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, out: torch.Tensor, eps: float) -> torch.Tensor:
+    """out = a N(z) + b N(z^2) + c N(z^3) + e, (a, b, c, e) = coef (float32 [4] on the device), N(v) = v / sqrt(mean(v^2) + eps)
+    over a row; z float32 [T, F]."""
+    _gpu(z, coef, out)
+    _need(z.dtype == torch.float32 and z.dim() == 2 and z.is_contiguous(), "poly_norm: z is contiguous float32 [T, F]")
+    _need(coef.dtype == torch.float32 and coef.numel() == 4 and coef.is_contiguous(), "poly_norm: four float32 coefficients")
+    _need(out.shape == z.shape and out.is_contiguous(), "poly_norm: out has z's shape")
+    _need(eps > 0, "poly_norm: eps must be positive")
+    _check(library().tm_poly_norm(_p(z), _p(coef), _p(out), c_int(code(out.dtype)), c_int(z.shape[0]), c_int(z.shape[1]),
+                                  c_float(eps), _stream()), "poly_norm")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- attention over a shared latent
+
+def _check_latent_pool(pool: torch.Tensor, Dk: int, dtype, who: str) -> int:
+    """The cached rows [pages, page, 1, Dk]; returns the page size."""
+    _need(pool.dim() == 4 and pool.is_contiguous() and pool.shape[2] == 1 and pool.shape[3] == Dk and pool.dtype == dtype,
+          f"{who}: the pool must be contiguous [pages, page, 1, {Dk}] of type {dtype}")
+    return pool.shape[1]
+
+
+def _angles(cos, sin, rot: int, positions, T: int, who: str) -> None:
+    if rot:
+        _need(cos is not None and sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32
+              and cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == rot // 2 and cos.is_contiguous() and sin.is_contiguous(),
+              f"{who}: cos/sin float32 [positions, {rot // 2}]")
+        _ints(positions, T, "positions")
+
+
+def latent_prepare(low: torch.Tensor, Lq: int, Lk: int, Dr: int, wq: torch.Tensor | None, wk: torch.Tensor, eps: float,
+                   cos: torch.Tensor | None, sin: torch.Tensor | None, positions: torch.Tensor | None, slots: torch.Tensor | None,
+                   cq: torch.Tensor | None, pool: torch.Tensor | None) -> None:
+    """low float32 [T, >= Lq + Lk + Dr] = [query latent | key/value latent | shared key]: cq [T, Lq] = rms_norm(query latent) * wq;
+    the cache row of token t (slot slots[t] of pool; < 0: not stored) = [rms_norm(latent) * wk | shared key with its first
+    2 * cos.shape[1] channels rotated in pairs (2i, 2i + 1) by the token's position]."""
+    _gpu(low, wq, wk, cos, sin, positions, slots, cq, pool)
+    T = low.shape[0]
+    _need(low.dtype == torch.float32 and low.dim() == 2 and low.stride(1) == 1 and low.shape[1] >= Lq + Lk + Dr,
+          f"latent_prepare: low is float32 [T, >= {Lq + Lk + Dr}]")
+    _need(wk.dtype == torch.float32 and tuple(wk.shape) == (Lk,) and wk.is_contiguous(), f"latent_prepare: wk is float32 [{Lk}]")
+    dt = None
+    if Lq:
+        _need(wq is not None and wq.dtype == torch.float32 and tuple(wq.shape) == (Lq,) and wq.is_contiguous(),
+              f"latent_prepare: wq is float32 [{Lq}]")
+        _need(cq is not None and tuple(cq.shape) == (T, Lq) and cq.is_contiguous(), f"latent_prepare: cq is contiguous [T, {Lq}]")
+        dt = cq.dtype
+    rot = 2 * cos.shape[1] if cos is not None else 0
+    _need(rot <= Dr, "latent_prepare: more rotated channels than the shared key has")
+    _angles(cos, sin, rot, positions, T, "latent_prepare")
+    if slots is not None:
+        _need(pool is not None, "latent_prepare: slots without a pool")
+        _check_latent_pool(pool, Lk + Dr, dt or pool.dtype, "latent_prepare")
+        dt = pool.dtype
+        _ints(slots, T, "slots")
+    _need(dt is not None, "latent_prepare: nothing to do")
+    ld = low.stride(0) if T > 1 else max(low.stride(0), low.shape[1])
+    _check(library().tm_latent_prepare(_p(low), c_int(ld), c_int(Lq), c_int(Lk), c_int(Dr), c_int(rot), _p(wq), _p(wk), c_float(eps),
+                                       _p(cos), _p(sin), _p(positions), _p(slots), _p(cq), _p(pool if slots is not None else None),
+                                       c_int(code(dt)), c_int(T), _stream()), "latent_prepare")
+
+
+def heads_matmul(a: torch.Tensor, a_head: int, b: torch.Tensor, c: torch.Tensor, c_head: int,
+                 gate: torch.Tensor | None = None) -> torch.Tensor:
+    """c[t, h * c_head + n] = sum_k a[t, h * a_head + k] * b[h, k, n] for n < N, k < K (b [H, K, N]); with ``gate`` (float32
+    [T, >= H], rows may be strided) the result is multiplied by sigmoid(gate[t, h]). a, b, c share one type; rows may be strided."""
+    _gpu(a, b, c, gate)
+    T = a.shape[0]
+    H, K, N = b.shape
+    _need(a.dim() == 2 and c.dim() == 2 and a.stride(1) == 1 and c.stride(1) == 1 and c.shape[0] == T and b.is_contiguous(),
+          "heads_matmul: a, c [T, .] with unit inner stride, b contiguous [H, K, N]")
+    _need(a.dtype == b.dtype == c.dtype, "heads_matmul: one type")
+    _need(a_head >= K and c_head >= N and a.shape[1] >= (H - 1) * a_head + K and c.shape[1] >= (H - 1) * c_head + N,
+          "heads_matmul: the heads do not fit the rows")
+    gate_stride = 0
+    if gate is not None:
+        _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= H and gate.stride(1) == 1,
+              "heads_matmul: gate is float32 [T, >= H]")
+        gate_stride = gate.stride(0) if T > 1 else max(gate.stride(0), H)
+    lda = a.stride(0) if T > 1 else max(a.stride(0), a.shape[1])
+    ldc = c.stride(0) if T > 1 else max(c.stride(0), c.shape[1])
+    _check(library().tm_heads_matmul(_p(a), c_int(lda), c_int(a_head), _p(b), _p(c), c_int(ldc), c_int(c_head), _p(gate),
+                                     c_int(gate_stride), c_int(T), c_int(H), c_int(K), c_int(N), c_int(code(a.dtype)), _stream()),
+           "heads_matmul")
+    return c
+
+
+def rotate_heads(src: torch.Tensor, src_head: int, dst: torch.Tensor, dst_head: int, H: int, Dr: int, cos: torch.Tensor | None,
+                 sin: torch.Tensor | None, positions: torch.Tensor | None) -> None:
+    """dst[t, h * dst_head + c] = src[t, h * src_head + c] for c < Dr, the first 2 * cos.shape[1] channels of every head rotated in
+    pairs (2i, 2i + 1) by the token's position. src and dst are views that start at the heads' first rotated channel."""
+    _gpu(src, dst, cos, sin, positions)
+    T = src.shape[0]
+    _need(src.dim() == 2 and dst.dim() == 2 and src.stride(1) == 1 and dst.stride(1) == 1 and dst.shape[0] == T and src.dtype == dst.dtype,
+          "rotate_heads: src, dst [T, .] of one type with unit inner stride")
+    _need(src_head >= Dr and dst_head >= Dr and src.shape[1] >= (H - 1) * src_head + Dr and dst.shape[1] >= (H - 1) * dst_head + Dr,
+          "rotate_heads: the heads do not fit the rows")
+    rot = 2 * cos.shape[1] if cos is not None else 0
+    _need(rot <= Dr, "rotate_heads: more rotated channels than a head has")
+    _angles(cos, sin, rot, positions, T, "rotate_heads")
+    lds = src.stride(0) if T > 1 else max(src.stride(0), src.shape[1])
+    ldd = dst.stride(0) if T > 1 else max(dst.stride(0), dst.shape[1])
+    _check(library().tm_rotate_heads(_p(src), c_int(lds), c_int(src_head), _p(dst), c_int(ldd), c_int(dst_head), c_int(T), c_int(H),
+                                     c_int(Dr), c_int(rot), _p(cos), _p(sin), _p(positions), c_int(code(src.dtype)), _stream()),
+           "rotate_heads")
+
+
+LATENT_MAX_ROW, LATENT_MAX_RANK = 704, 512
+
+
+def attn_latent(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, block_tables: torch.Tensor, seq_of_token: torch.Tensor,
+                positions: torch.Tensor, H: int, Lk: int, Dk: int, scale: float, window: int = 0) -> torch.Tensor:
+    """out[t, h, :Lk] = sum_j softmax_j(scale * qa[t, h, :Dk] . row[j]) * row[j, :Lk] over the cached rows j of the token's
+    request with 0 <= position - j < window (0: every row up to the token's own). qa [T, H * Dk], out [T, H * Lk]."""
+    _gpu(qa, out, pool, block_tables, seq_of_token, positions)
+    T = qa.shape[0]
+    _need(qa.is_contiguous() and tuple(qa.shape) == (T, H * Dk) and out.is_contiguous() and tuple(out.shape) == (T, H * Lk)
+          and qa.dtype == out.dtype, f"attention(latent): qa [T, {H * Dk}] and out [T, {H * Lk}] contiguous, of one type")
+    _need(0 < Lk <= Dk <= LATENT_MAX_ROW and Lk <= LATENT_MAX_RANK, f"attention(latent): rows of up to {LATENT_MAX_ROW} with a latent of up to {LATENT_MAX_RANK}")
+    page = _check_latent_pool(pool, Dk, qa.dtype, "attention(latent)")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "attention(latent): block_tables must be contiguous int32 [S, W]")
+    _ints(seq_of_token, T, "seq_of_token")
+    _ints(positions, T, "positions")
+    _need(window >= 0, "attention(latent): window must be >= 0")
+    _check(library().tm_attn_latent(_p(qa), c_int(H * Dk), _p(out), c_int(H * Lk), _p(pool), _p(block_tables), c_int(block_tables.shape[1]),
+                                    _p(seq_of_token), _p(positions), c_int(T), c_int(H), c_int(Lk), c_int(Dk), c_int(page),
+                                    c_float(scale), c_int(window), c_int(code(qa.dtype)), _stream()), "attn_latent")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- experts by table
+
+MOE_TILE_ROWS = 32
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_max_tiles(pairs: int, experts: int) -> int:
+    """The most tiles of MOE_TILE_ROWS rows that ``pairs`` (token, expert) pairs can fall into."""
+    return min(pairs, pairs // MOE_TILE_ROWS + experts)
+
+
+def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int):
+    """Sorts the step's (token, choice) pairs by expert. Returns int32 tensors (slot_pair [P], pair_slot [P], tiles [max, 3],
+    n_tiles [1]); see ``csrc/moe.hip``."""
+    _gpu(token_ids, table)
+    T = token_ids.numel()
+    _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "moe_route: table is contiguous int32 [vocab, top]")
+    _ints(token_ids, T, "token_ids")
+    top = table.shape[1]
+    _need(0 < experts <= MOE_MAX_EXPERTS, f"moe_route: up to {MOE_MAX_EXPERTS} experts")
+    P = T * top
+    most = moe_max_tiles(P, experts)
+    work = torch.empty(2 * P + 3 * most + 1, dtype=torch.int32, device=token_ids.device)
+    slot_pair, pair_slot, tiles, n_tiles = work[:P], work[P:2 * P], work[2 * P:2 * P + 3 * most].view(most, 3), work[2 * P + 3 * most:]
+    _check(library().tm_moe_route(_p(token_ids), _p(table), c_int(T), c_int(top), c_int(experts), c_int(MOE_TILE_ROWS), _p(slot_pair),
+                                  _p(pair_slot), _p(tiles), _p(n_tiles), _stream()), "moe_route")
+    return slot_pair, pair_slot, tiles, n_tiles
+
+
+def moe_experts(x: torch.Tensor, routed, w_gate_up: torch.Tensor, w_down: torch.Tensor, top: int, weight: float,
+                out: torch.Tensor) -> torch.Tensor:
+    """out[t] = sum over the token's ``top`` experts e of weight * Wd[e] (silu(Wg[e] x[t]) * (Wu[e] x[t])), in the order of
+    its choices. w_gate_up [E, 2F, K] (gate rows, then up rows), w_down [E, N, F]; ``routed`` from ``moe_route``."""
+    slot_pair, pair_slot, tiles, n_tiles = routed
+    _gpu(x, w_gate_up, w_down, out)
+    T, K = x.shape
+    E, F2, K2 = w_gate_up.shape
+    F = F2 // 2
+    N = w_down.shape[1]
+    P = T * top
+    _need(x.stride(1) == 1 and K2 == K and F2 == 2 * F and tuple(w_down.shape) == (E, N, F) and w_gate_up.is_contiguous()
+          and w_down.is_contiguous(), "moe_experts: x [T, K], w_gate_up [E, 2F, K], w_down [E, N, F]")
+    _need(x.dtype == w_gate_up.dtype == w_down.dtype == out.dtype, "moe_experts: one type")
+    _need(tuple(out.shape) == (T, N) and out.is_contiguous(), f"moe_experts: out is contiguous [{T}, {N}]")
+    _need(slot_pair.numel() == P and pair_slot.numel() == P, "moe_experts: the routing belongs to another step")
+    most = tiles.shape[0]
+    act = torch.empty((P, F), dtype=x.dtype, device=x.device)
+    part = torch.empty((P, N), dtype=torch.float32, device=x.device)
+    lib, dt = library(), c_int(code(x.dtype))
+    ldx = x.stride(0) if T > 1 else max(x.stride(0), K)
+    _check(lib.tm_moe_gate_up(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_gate_up), _p(act), _p(tiles), _p(n_tiles), c_int(most),
+                              c_int(K), c_int(F), dt, _stream()), "moe_gate_up")
+    _check(lib.tm_moe_down(_p(act), _p(w_down), _p(part), _p(tiles), _p(n_tiles), c_int(most), c_int(F), c_int(N), dt, _stream()),
+           "moe_down")
+    _check(lib.tm_moe_combine(_p(part), _p(pair_slot), _p(out), c_int(T), c_int(top), c_float(weight), c_int(N), dt, _stream()),
+           "moe_combine")
+    return out

@@ -146,7 +146,7 @@ class StepProgram:
         """resid += o(attention(rotate(qkv(norm(resid))))) over the paged cache ``cache`` (a ``KVCacheView``).
         ``rotation``: (cos, sin, rotary width, positions) of a rotary encoding, or () for none."""
         n, q, out = self._norm(norm), self._linear(qkv), self._linear(o)
-        if n is None or q is None or out is None or getattr(cache, "k", None) is None:
+        if n is None or q is None or out is None or getattr(cache, "k", None) is None or getattr(cache, "v", None) is None:
             return None
         if rotation:
             cos, sin, rot, n_pos = rotation

@@ -39,7 +39,7 @@ class DecoderModel:
             if call.cache_of is not None:
                 if not 0 <= call.cache_of < j or self.run[call.cache_of].cache_of is not None:
                     raise ValueError(f"run[{j}] must read the cache of an earlier call that owns one")
-                if layers[call.layer].mixer.cache_spec() != layers[self.run[call.cache_of].layer].mixer.cache_spec():
+                if self._cache_spec(layers[call.layer]) != self._cache_spec(layers[self.run[call.cache_of].layer]):
                     raise ValueError(f"run[{j}] reads a cache of another geometry than its own mixer's")
 
     # --- tensors ---------------------------------------------------------------------------------
@@ -70,7 +70,12 @@ class DecoderModel:
 
     def cache_specs(self) -> list[KVCacheSpec | StateSpec | None]:
         """One entry per run call: the cache its mixer needs, or None for a call that reads another's."""
-        return [None if c.cache_of is not None else self.layers[c.layer].mixer.cache_spec() for c in self.run]
+        return [None if c.cache_of is not None else self._cache_spec(self.layers[c.layer]) for c in self.run]
+
+    @staticmethod
+    def _cache_spec(layer):
+        # a layer says what it needs; one that does not (a block written elsewhere) is asked through its mixer
+        return layer.cache_spec() if hasattr(layer, "cache_spec") else layer.mixer.cache_spec()
 
     # --- one step -----------------------------------------------------------------------------------
 

@@ -24,16 +24,18 @@ from tokenmill_amd.weights.loader import TensorSpec
 class KVCacheSpec:
     """Keys and values in pages. ``window``: None keeps every token; W keeps the last W. ``chunk``: C means that a
     token never reads a key from before the start of its own chunk of C positions (counted from position 0), so the
-    pages of finished chunks can be given back. ``v_head_dim``: size of a value where it differs from a key's."""
+    pages of finished chunks can be given back. ``v_head_dim``: size of a value where it differs from a key's.
+    ``values``: False for a mixer whose values are part of its key rows (a shared latent): the group has no value pool."""
     kv_heads: int
     head_dim: int
     window: int | None = None
     v_head_dim: int | None = None
     chunk: int | None = None
+    values: bool = True
 
     @property
     def value_dim(self) -> int:
-        return self.v_head_dim or self.head_dim
+        return (self.v_head_dim or self.head_dim) if self.values else 0
 
     def first_needed(self, num_computed: int) -> int:
         """With ``num_computed`` tokens cached, the next query sits at position num_computed or later: the first
@@ -52,18 +54,27 @@ class KVCacheSpec:
 
 @dataclass(frozen=True)
 class StateSpec:
-    """State of fixed size per request (zeroed when a request is admitted)."""
+    """State of fixed size per request (zeroed when a request is admitted). ``dtype`` None: the model's storage type."""
     shape: tuple[int, ...]
-    dtype: torch.dtype = torch.float32
+    dtype: torch.dtype | None = torch.float32
+
+
+@dataclass(frozen=True)
+class LayerCacheSpec:
+    """What a layer needs when it is more than one thing: pages for its mixer's keys and a slot of state beside them
+    (a short convolution in front of an attention). Either may be None."""
+    kv: KVCacheSpec | None = None
+    state: StateSpec | None = None
 
 
 @dataclass
 class KVCacheView:
     """One cache layer as a mixer sees it."""
     k: torch.Tensor              # [pages, page_size, kv_heads, head_dim]
-    v: torch.Tensor              # [pages, kv_heads, value size, page_size]
+    v: torch.Tensor | None       # [pages, kv_heads, value size, page_size]; None for a group without a value pool
     group: int                   # index into StepContext.groups
     write: bool = True           # False: this layer reads a cache that another layer writes
+    state: torch.Tensor | None = None    # [slots, *shape] of a layer that keeps state beside its pages
 
 
 @dataclass
@@ -255,6 +266,10 @@ class Block(Part):
     default as one call of ``forward``, so a block written elsewhere needs nothing more."""
 
     mixer: Mixer
+
+    def cache_spec(self):
+        """What the layer asks of the cache manager: its mixer's needs, unless the block keeps something itself."""
+        return self.mixer.cache_spec()
 
     def forward(self, resid: torch.Tensor, delta: torch.Tensor | None, step: StepContext, cache,
                 dtype: torch.dtype) -> torch.Tensor | None:

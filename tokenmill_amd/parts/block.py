@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from tokenmill_amd.parts.base import Block, FeedForward, Mixer, Norm, NormedInput, StepContext
+from tokenmill_amd.parts.base import Block, FeedForward, LayerCacheSpec, Mixer, Norm, NormedInput, StepContext
 
 
 class PreNormBlock(Block):
@@ -124,4 +124,103 @@ class SandwichBlock(Block):
             return None
         y = self.ffn.forward(NormedInput(self.norm_post, resid, y, dtype, delta_norm=self.norm_mixed), step)
         self.norm_fed.add_normed(resid, y)
+        return None
+
+
+class GatedResidualBlock(Block):
+    """Pre-norm sublayers whose results are scaled and gated on their way into the residual stream:
+
+        n = norm_in(x);    x += mult * mixer(n + conv(n)) * sigmoid(gate_mixed(n))
+        n = norm_post(x);  x += mult * ffn(n) * sigmoid(gate_fed(n))             (only with a feed-forward)
+
+    ``conv`` (a ``ShortConvolution`` in front of the mixer), the two gates (``Linear`` parts with a bias) and the
+    feed-forward are each optional, and ``mult`` = 1 with no gate is the plain pre-norm block. A gate reads the normed
+    input before the convolution. A sublayer's result stays pending with its gate (``GatedAdd``) so that the norm in front
+    of the next sublayer, of this block or the next, adds it and norms the sum in one kernel. The convolution's state lies
+    beside the mixer's pages in the layer's cache."""
+
+    def __init__(self, norm_in: Norm, mixer: Mixer, norm_post: Norm | None = None, ffn: FeedForward | None = None,
+                 gate_mixed=None, gate_fed=None, conv=None, mult: float = 1.0,
+                 names: tuple[str, str, str, str] = ("norm1", "mix.", "norm2", "mlp.")):
+        if (ffn is None) != (norm_post is None):
+            raise ValueError("a feed-forward comes with the norm before it, or not at all")
+        if ffn is None and gate_fed is not None:
+            raise ValueError("a gate for a feed-forward that is not there")
+        self.norm_in, self.mixer, self.norm_post, self.ffn = norm_in, mixer, norm_post, ffn
+        self.gate_mixed, self.gate_fed, self.conv, self.mult = gate_mixed, gate_fed, conv, float(mult)
+        self.names = names
+
+    def _parts(self):
+        # the gates and the convolution carry their own names and take the layer's prefix
+        pairs = list(zip((self.norm_in, self.mixer, self.norm_post, self.ffn), self.names))
+        pairs += [(self.gate_mixed, ""), (self.gate_fed, ""), (self.conv, "")]
+        return [(p, n) for p, n in pairs if p is not None]
+
+    def tensor_specs(self, prefix: str):
+        specs = {}
+        for part, name in self._parts():
+            specs.update(part.tensor_specs(prefix + name))
+        return specs
+
+    def load(self, tensors, prefix: str) -> None:
+        for part, name in self._parts():
+            part.load(tensors, prefix + name)
+
+    def prepare(self, pack_weights: bool) -> None:
+        for part, _ in self._parts():
+            part.prepare(pack_weights)
+
+    def cache_spec(self):
+        spec = self.mixer.cache_spec()
+        state = self.conv.state_spec() if self.conv is not None else None
+        if state is None:
+            return spec
+        if spec is not None and not hasattr(spec, "kv_heads"):
+            raise ValueError("a convolution in front of a mixer that keeps state of its own is not arranged for")
+        return LayerCacheSpec(spec, state)
+
+    def _pending(self, gate):
+        from tokenmill_amd.parts.norm import GatedAdd
+        return GatedAdd(gate, self.mult) if gate is not None or self.mult != 1.0 else None
+
+    def _gate(self, part, n):
+        from tokenmill_amd import profiling
+        if part is None:
+            return None
+        with profiling.label("gate", lambda: part.cost(n.shape[0])):
+            return part.forward(n)
+
+    def _mix(self, x: NormedInput, step: StepContext, cache):
+        n = x.tensor()
+        gate = self._gate(self.gate_mixed, n)
+        u = self.conv.forward(n, step, getattr(cache, "state", None)) if self.conv is not None else n
+        return self.mixer.forward(u, step, cache), self._pending(gate)
+
+    def _feed(self, x: NormedInput, step: StepContext):
+        n = x.tensor()
+        gate = self._gate(self.gate_fed, n)
+        return self.ffn.forward(n, step), self._pending(gate)
+
+    def emit(self, program, cache) -> None:
+        def mix(flow, step):
+            x = NormedInput(self.norm_in, flow.resid, flow.delta, program.dtype, delta_norm=flow.delta_norm)
+            flow.delta, flow.delta_norm = self._mix(x, step, cache)
+        program.foreign(self.mixer, mix)
+        if self.ffn is not None:
+            def feed(flow, step):
+                x = NormedInput(self.norm_post, flow.resid, flow.delta, program.dtype, delta_norm=flow.delta_norm)
+                flow.delta, flow.delta_norm = self._feed(x, step)
+            program.foreign(self.ffn, feed)
+
+    def forward(self, resid: torch.Tensor, delta: torch.Tensor | None, step: StepContext, cache,
+                dtype: torch.dtype) -> None:
+        """The block by itself: resid float32 [T, hidden] is updated in place with everything; nothing is left pending."""
+        y, way = self._mix(NormedInput(self.norm_in, resid, delta, dtype), step, cache)
+        if self.ffn is not None:
+            y, way = self._feed(NormedInput(self.norm_post, resid, y, dtype, delta_norm=way), step)
+        if way is not None:
+            way.add_normed(resid, y)
+        else:
+            from tokenmill_amd.parts.norm import GatedAdd
+            GatedAdd(None, 1.0).add_normed(resid, y)
         return None

@@ -8,6 +8,7 @@ from tokenmill_amd.hip import ops
 from tokenmill_amd.hip.program import StepProgram
 from tokenmill_amd.parts.base import FeedForward, Norm, NormedInput, StepContext, as_tensor
 from tokenmill_amd.parts.linear import Linear
+from tokenmill_amd.weights.loader import TensorSpec
 
 
 class SwiGLU(FeedForward):
@@ -68,25 +69,35 @@ class SwiGLU(FeedForward):
 
 
 class DenseFeedForward(FeedForward):
-    """down(act(up(x))) with one up matrix and no gate; ``activation``: "gelu_tanh", the tanh form of GELU,
-    0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), computed in 32-bit. Both products may have biases."""
+    """down(act(up(x))) with one up matrix and no gate. ``activation``: "gelu_tanh", the tanh form of GELU,
+    0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))); or "poly_norm", a N(z) + b N(z^2) + c N(z^3) + e with four learned
+    numbers (a, b, c, e) (the tensor ``act_name``), powers taken element by element and N(v) = v / sqrt(mean(v^2) + eps)
+    over a token's row (``act_eps``). Both are computed in 32-bit. Both products may have biases."""
 
-    ACTIVATIONS = {"gelu_tanh": ops.gelu_tanh}
+    ACTIVATIONS = ("gelu_tanh", "poly_norm")
 
     def __init__(self, hidden: int, intermediate: int, activation: str = "gelu_tanh", bias: bool = True,
-                 names: tuple[str, str] = ("up", "down"), suffixes: tuple[str, str] = (".weight", ".bias")):
+                 names: tuple[str, str] = ("up", "down"), suffixes: tuple[str, str] = (".weight", ".bias"),
+                 act_name: str = "act", act_eps: float = 1e-6):
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"activation '{activation}' is not one of {sorted(self.ACTIVATIONS)}")
         self.hidden, self.intermediate, self.activation = hidden, intermediate, activation
         self.up = Linear(hidden, intermediate, names[0], bias=bias, suffixes=suffixes)
         self.down = Linear(intermediate, hidden, names[1], bias=bias, suffixes=suffixes)
+        self.act_name, self.act_eps = act_name, float(act_eps)
+        self.act: torch.Tensor | None = None        # the activation's learned numbers, 32-bit
 
     def tensor_specs(self, prefix: str):
-        return {**self.up.tensor_specs(prefix), **self.down.tensor_specs(prefix)}
+        specs = {**self.up.tensor_specs(prefix), **self.down.tensor_specs(prefix)}
+        if self.activation == "poly_norm":
+            specs[prefix + self.act_name] = TensorSpec((4,), init="ones")
+        return specs
 
     def load(self, tensors, prefix: str) -> None:
         self.up.load(tensors, prefix)
         self.down.load(tensors, prefix)
+        if self.activation == "poly_norm":
+            self.act = tensors[prefix + self.act_name].float().contiguous()
 
     def cost(self, label: str, step: StepContext | None, rows: int) -> tuple[int, int]:
         return self.up.cost(rows) if label == "gate_up" else self.down.cost(rows)
@@ -95,7 +106,11 @@ class DenseFeedForward(FeedForward):
         from tokenmill_amd import profiling
         x = as_tensor(x)
         with profiling.label("gate_up", lambda: self.up.cost(x.shape[0])):
-            a = self.up.forward(x)
-            self.ACTIVATIONS[self.activation](a, a)
+            if self.activation == "poly_norm":          # the row's statistics want the products' sums as they are
+                z = self.up.forward(x, out_dtype=torch.float32)
+                a = ops.poly_norm(z, self.act, torch.empty(z.shape, dtype=x.dtype, device=x.device), self.act_eps)
+            else:
+                a = self.up.forward(x)
+                ops.gelu_tanh(a, a)
         with profiling.label("down", lambda: self.down.cost(x.shape[0])):
             return self.down.forward(a)

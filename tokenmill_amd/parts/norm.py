@@ -81,3 +81,59 @@ class GroupRMSNorm(Norm):
     def add_normed(self, resid, y) -> None:
         with profiling.label("norm", lambda: self._cost(resid.shape[0], 4, y.element_size())):
             ops.group_norm(resid, y, self.weight, None, None, self.groups, self.eps)
+
+
+class GatedAdd:
+    """What a sublayer's result passes on its way into the residual stream when the block scales and gates it:
+    resid += mult * y * sigmoid(gate), with ``gate`` [T, hidden] the gate's values before the sigmoid (None: no gate).
+    It stands where a norm behind a sublayer stands (``Flow.delta_norm``), so the norm in front of the next sublayer
+    can do the add and its own work in one kernel."""
+
+    def __init__(self, gate: torch.Tensor | None, mult: float = 1.0):
+        self.gate, self.mult = gate, float(mult)
+
+    def add_normed(self, resid, y) -> None:
+        with profiling.label("norm", lambda: (resid.numel() * 8 + y.numel() * y.element_size() * (2 if self.gate is not None else 1), 0)):
+            ops.layer_norm(resid, y, self.gate, self.mult, None, None, None, 1.0)
+
+
+class LayerNorm(Norm):
+    """(x - mean) / sqrt(mean((x - mean)^2) + eps) * weight + bias over a row, in 32-bit, rounded once. The weight and
+    the bias are kept in 32-bit. ``names``: what the checkpoint appends to the prefix for the two."""
+
+    def __init__(self, hidden: int, eps: float, names: tuple[str, str] = ("weight", "bias")):
+        self.hidden, self.eps, self.names = hidden, float(eps), names
+        self.weight: torch.Tensor | None = None
+        self.bias: torch.Tensor | None = None
+
+    def tensor_specs(self, prefix: str):
+        return {prefix + self.names[0]: TensorSpec((self.hidden,), init="ones"),
+                prefix + self.names[1]: TensorSpec((self.hidden,), init="zeros")}
+
+    def load(self, tensors, prefix: str) -> None:
+        self.weight = tensors[prefix + self.names[0]].float().contiguous()
+        self.bias = tensors[prefix + self.names[1]].float().contiguous()
+
+    def _cost(self, n: int, out_bytes: int, added: int):
+        return n * self.hidden * (4 + out_bytes + added), 0
+
+    def add_norm(self, resid, delta, out_dtype, rows=None, delta_norm=None):
+        n = resid.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.hidden), dtype=out_dtype, device=resid.device)
+        gate, mult = None, 1.0
+        if delta is not None and delta_norm is not None:
+            if isinstance(delta_norm, GatedAdd):
+                gate, mult = delta_norm.gate, delta_norm.mult
+            elif rows is None:
+                delta_norm.add_normed(resid, delta)
+                delta = None
+            else:       # only some rows are wanted and the residual is to stay as it is: the pending result's way in on a copy
+                resid = resid.index_select(0, rows.long())
+                delta_norm.add_normed(resid, delta.index_select(0, rows.long()))
+                delta, rows = None, None
+        added = 0 if delta is None else (4 if rows is None else 0) + delta.element_size() * (2 if gate is not None else 1)
+        with profiling.label("norm", lambda: self._cost(n, out.element_size(), added)):
+            return ops.layer_norm(resid, delta, gate, mult, self.weight, self.bias, out, self.eps, rows)
+
+    def add_normed(self, resid, y) -> None:
+        raise NotImplementedError("a layer norm stands in front of a sublayer, not behind it")

@@ -13,10 +13,14 @@ from tokenmill_amd.parts.base import KVCacheView, PositionEncoding, StepContext
 
 
 class RotaryEmbedding(PositionEncoding):
-    """Pairs (j, j + rotary_dim/2) of each head rotate by position * theta^(-2j/rotary_dim)."""
+    """Pairs (j, j + rotary_dim/2) of each head rotate by position * theta^(-2j/rotary_dim). ``interleaved``: the pairs
+    are the neighbours (2j, 2j + 1) instead; the table of angles is the same, and a mixer that wants that pairing rotates
+    with kernels of its own (the kernel library's attention operation knows the first pairing only)."""
 
-    def __init__(self, head_dim: int, theta: float, max_positions: int, rotary_dim: int | None = None):
+    def __init__(self, head_dim: int, theta: float, max_positions: int, rotary_dim: int | None = None,
+                 interleaved: bool = False):
         self.head_dim = head_dim
+        self.interleaved = interleaved
         self.rotary_dim = rotary_dim or head_dim
         if self.rotary_dim % 2 or self.rotary_dim > head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {head_dim}")
@@ -38,6 +42,8 @@ class RotaryEmbedding(PositionEncoding):
             self.build_tables(device)
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, step: StepContext, cache: KVCacheView | None):
+        if self.interleaved:
+            raise NotImplementedError("neighbouring pairs are rotated by the mixer that asked for them")
         if step.max_context_len > self.max_positions:
             raise ValueError(f"position {step.max_context_len - 1} is beyond the rotary table "
                              f"({self.max_positions} positions)")
@@ -48,6 +54,8 @@ class RotaryEmbedding(PositionEncoding):
 
     def rotation(self):
         """(cos, sin, rotary width, positions): what the kernel library's attention operation rotates by."""
+        if self.interleaved:
+            return None
         return (self.cos, self.sin, self.rotary_dim, self.max_positions) if self.cos is not None else None
 
 

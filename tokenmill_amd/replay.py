@@ -99,7 +99,7 @@ def main(argv=None) -> int:
     p.add_argument("--out", required=True, help="folder for <step>.f32 files")
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens live requests hold at any time (each rounded up to a multiple of 64)")
-    p.add_argument("--max-requests", type=int, default=16, help="most requests live at a time")
+    p.add_argument("--max-requests", type=int, default=4, help="most requests live at a time")
     p.add_argument("--block-size", type=int, default=PAGE_SIZE, help="tokens per cache page")
     args = p.parse_args(argv)
 

@@ -27,7 +27,7 @@ class TensorSpec:
     when the tensor is drawn at random."""
     shape: tuple[int | None, ...]
     kind: str = "float"          # "float" | "int"
-    init: str = "normal"         # random-weights mode: "normal" | "ones" | "zeros" | "index"
+    init: str = "normal"         # random-weights mode: "normal" | "ones" | "zeros" | "index" | "distinct_below:N" (int rows of different numbers < N)
     free: tuple[int, ...] = ()
 
     def fits(self, got: tuple[int, ...]) -> bool:

@@ -27,6 +27,12 @@ def _generator(seed: int, name: str) -> torch.Generator:
     return torch.Generator().manual_seed(int.from_bytes(digest[:8], "little") >> 1)
 
 
+def distinct_rows(shape: tuple[int, ...], below: int, g: torch.Generator, device=None) -> torch.Tensor:
+    """An int32 table [rows, k] whose rows each hold k different numbers below ``below``, in random order."""
+    rows, k = shape
+    return torch.rand((rows, below), generator=g, device=device).argsort(dim=1)[:, :k].to(torch.int32).contiguous()
+
+
 def random_tensors(specs: dict[str, TensorSpec], seed: int, std: float = 0.02, norm_std: float = 0.0,
                    storage: torch.dtype = torch.bfloat16) -> Iterator[tuple[str, torch.Tensor]]:
     """(name, tensor) for every spec: "normal" ~ N(0, std); "ones" = 1 + N(0, norm_std)."""
@@ -34,7 +40,9 @@ def random_tensors(specs: dict[str, TensorSpec], seed: int, std: float = 0.02, n
         spec = specs[name]
         shape = spec.drawn_shape()
         g = _generator(seed, name)
-        if spec.kind == "int":
+        if spec.kind == "int" and spec.init.startswith("distinct_below:"):
+            t = distinct_rows(shape, int(spec.init.split(":")[1]), g)
+        elif spec.kind == "int":
             t = torch.arange(int(torch.tensor(shape).prod()), dtype=torch.int32).reshape(shape)
         elif spec.init == "ones":
             t = torch.ones(shape, dtype=torch.float32)
