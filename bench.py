@@ -3,7 +3,7 @@ weights, synthetic token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
                     [--config CONFIG.json|NAME]      another shape of the architecture (7b, 32b, a file)
-                    [--part all|decode|prefill|offline|mixed7b|preempt32b|modinex]
+                    [--part all|decode|prefill|offline|mixed7b|preempt32b|modinex|lusolix]
                     [--part decode --contexts 8192,32768 --batches 8,64]     decode steps over long contexts
 
 A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
@@ -19,6 +19,7 @@ of their operations has to move and do), not from formulas of one architecture.
                         (portions of prompts beside decoding requests, budget 2,048), up to 64 at a time
     --part preempt32b   the 32B shape, context 8,192: 64 prompts of 2,048 ids on 8,192 pages of 16, so
                         that growth during decoding evicts requests; reports evictions and tok/s
+    --part lusolix      the Lusolix design at two such sizes (lusolix-1k, lusolix-2k) beside the same two Qwen2 models
     --part modinex      the Modinex design at two sizes that resemble a real model's layers (shipped shapes modinex-1k,
                         modinex-2k), each beside the Qwen2 model of equal width, depth, heads and feed-forward
                         parameters (qwen2-like-1k, qwen2-like-2k): prefill and decode rates, and per operation its
@@ -44,8 +45,19 @@ HISTOGRAM_STEPS = 128            # the step-time histogram is taken over at leas
 PROFILED_STEPS = 8               # decode steps run under the kernel trace
 
 
+class _Matrices:
+    """Matrices a part keeps outside Linear parts (per-head or per-expert stacks), counted like a Linear's."""
+
+    def __init__(self, tensors):
+        self._n = sum(t.numel() for t in tensors)
+        self.weight = self
+
+    def numel(self) -> int:
+        return self._n
+
+
 def _linears(model):
-    """Every Linear part of a model (for a count of its matrix parameters)."""
+    """Every Linear part of a model (for a count of its matrix parameters), and what a part says it keeps beside them."""
     from tokenmill_amd.parts import Linear
     seen, stack, out = set(), [model], []
     while stack:
@@ -60,6 +72,8 @@ def _linears(model):
             stack.extend(obj)
         elif hasattr(obj, "__dict__") and type(obj).__module__.startswith("tokenmill_amd"):
             stack.extend(vars(obj).values())
+            if hasattr(obj, "other_matrices"):
+                out.append(_Matrices(obj.other_matrices()))
     return out
 
 
@@ -87,7 +101,7 @@ def main() -> int:
                     help="captured shapes also try every algorithm the library holds, not only its heuristic's candidates")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
     ap.add_argument("--skip-kernels", action="store_true", help="no per-operation kernel trace")
-    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b", "modinex"],
+    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b", "modinex", "lusolix"],
                     help="all: the headline line. decode / prefill: only that (for profiling one of them). offline: "
                          "--requests prompts of --offline-prompt tokens submitted at once. mixed7b / preempt32b: see above")
     ap.add_argument("--requests", type=int, default=None, help="requests of the offline, mixed7b and preempt32b parts")
@@ -134,7 +148,7 @@ def main() -> int:
     # the position tables reach the longest context any engine of this run allows (each engine has its own limit)
     most_positions = max([max_model_len] + sweep + ([] if args.skip_points or args.part != "all" else list(LONG_POINTS)))
     most_positions = min(most_positions, shape.get("max_position_embeddings", most_positions))
-    model = None if args.part == "modinex" else load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
+    model = None if args.part in ("modinex", "lusolix") else load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
     gen = torch.Generator().manual_seed(0)
     vocab = model.head.vocab if model is not None else None
 
@@ -353,12 +367,12 @@ def main() -> int:
                 "config": {**sizes(), "requests": n, "prompt": prompt_len, "gen": gen_tokens, "max_num_seqs": n,
                            "token_budget": 2048, "max_model_len": max_model_len, "block_size": BLOCK_SIZE, "pages": pages}}
 
-    if args.part == "modinex":
+    if args.part in ("modinex", "lusolix"):
         # the new design beside the closest existing model at equal size: the functions above measure whatever
         # `model` is, so each shape is loaded in turn
         rows = {}
         for size in ("1k", "2k"):
-            for name in (f"modinex-{size}", f"qwen2-like-{size}"):
+            for name in (f"{args.part}-{size}", f"qwen2-like-{size}"):
                 shape, shape_name = read_shape(name), name
                 model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
                 vocab = model.head.vocab
@@ -376,7 +390,7 @@ def main() -> int:
                 del model
                 model = None
                 torch.cuda.empty_cache()
-        print(json.dumps({"metric": f"Modinex beside Qwen2 at equal size: prefill of {prompt_len} tokens, decode at batch {args.batch}",
+        print(json.dumps({"metric": f"{args.part.capitalize()} beside Qwen2 at equal size: prefill of {prompt_len} tokens, decode at batch {args.batch}",
                           "dtype": args.dtype, "prompt": prompt_len, "batch": args.batch, "rows": rows}))
         return 0
     if args.part == "offline":

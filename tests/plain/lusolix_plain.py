@@ -146,8 +146,10 @@ def forward(cfg: dict, t: dict, token_ids, dtype=torch.float32, start: int = 0, 
         L = f"l{i}."
         n = rnd(layer_norm(x, t[L + "norm1"], t[L + "norm1.b"], eps), dtype)
         g = torch.sigmoid(rnd(linear(n, t[L + "rg1"], t[L + "rg1.b"], dtype), dtype))
-        u, state[L + "conv"] = short_conv(n, t[L + "canon1"], state.get(L + "conv"))
-        u = rnd(u, dtype)
+        u = n
+        if L + "canon1" in t:
+            u, state[L + "conv"] = short_conv(n, t[L + "canon1"], state.get(L + "conv"))
+            u = rnd(u, dtype)
         y, state[L + "kv"] = latent_attention(u, pos, layer["mixer"], t, L + "mix.", eps, dtype, state.get(L + "kv"))
         x = x + mult * (rnd(y, dtype) * g)
         mlp = layer.get("mlp")

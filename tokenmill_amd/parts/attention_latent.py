@@ -88,6 +88,10 @@ class LatentAttention(Mixer):
     def cache_spec(self):
         return KVCacheSpec(1, self.row, self.window, values=False)
 
+    def other_matrices(self) -> list[torch.Tensor]:
+        """The matrices kept outside ``Linear`` parts (for a count of parameters)."""
+        return [self.uk, self.uv]
+
     def visible_pairs(self, step: StepContext) -> tuple[int, int]:
         """(rows read, (query, row) pairs) of a step, for a profile's floor."""
         rows = pairs = 0

@@ -57,6 +57,10 @@ class TableRoutedExperts(FeedForward):
                 raise ValueError(f"{prefix}{self.table_name}: a row names an expert twice")
         self.table = table.to(torch.int32).contiguous()
 
+    def other_matrices(self) -> list[torch.Tensor]:
+        """The matrices kept outside ``Linear`` parts (for a count of parameters)."""
+        return [self.gate_up, self.down]
+
     def cost(self, label: str, step: StepContext | None, rows: int) -> tuple[int, int]:
         e = self.gate_up.element_size()
         used = min(self.experts, rows * self.top)               # matrices read at least once each when every pair differs
