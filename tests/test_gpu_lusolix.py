@@ -263,7 +263,7 @@ def test_rows_just_inside_and_just_outside_the_window_show(dt, window, page):
     token's result is then, channel by channel, how many visible rows set that channel, over the number of visible rows.
     One row too many or too few, at the window's far edge or at the token itself, changes both."""
     from tokenmill_amd.hip import ops
-    H, Lk, Dr = 2, 40, 4
+    H, Lk, Dr = 5, 40, 8
     Dk = Lk + Dr
     n = 90
     pool = torch.zeros((n // page + 2, page, 1, Dk), dtype=dt, device=DEV)
@@ -273,15 +273,29 @@ def test_rows_just_inside_and_just_outside_the_window_show(dt, window, page):
         flat[int(table[j // page]) * page + j % page, j % Lk] = 1.0
     qa = torch.zeros((n, H * Dk), dtype=dt, device=DEV)                              # every score is zero
     out = torch.empty((n, H * Lk), dtype=dt, device=DEV)
-    ops.attn_latent(qa, out, pool, table.view(1, -1).to(DEV), ints([0] * n), ints(list(range(n))), H, Lk, Dk, 0.3, window)
-    got = out.float().cpu().view(n, H, Lk)
-    for p in range(n):
-        lo = max(0, p - window + 1)
-        want = torch.zeros(Lk)
-        for j in range(lo, p + 1):
-            want[j % Lk] += 1.0 / (p - lo + 1)
-        for h in range(H):
-            close(got[p, h], q(want, dt), dt, f"position {p} head {h}", bf16=2.0 ** -8)
+    tab = table.view(1, -1).to(DEV)
+    ops.attn_latent(qa, out, pool, tab, ints([0] * n), ints(list(range(n))), H, Lk, Dk, 0.3, window)
+    results = {"a wavefront a pair": out.float().cpu().view(n, H, Lk)}
+    if dt == torch.bfloat16:
+        # the matrix-unit kernel: the same rows as prompt tiles (the last one not full, one that starts inside a page), then as
+        # single tokens
+        assert ops.attn_latent_mfma_takes(dt, Lk, Dk, H)
+        cuts = [(0, 16), (16, 16), (32, 5), (37, 16), (53, 16), (69, 16), (85, 5)]
+        tiles = torch.tensor([[0, a, k, a] for a, k in cuts], dtype=torch.int32, device=DEV)
+        tiled = torch.full_like(out, math.nan)
+        ops.attn_latent_mfma(qa, tiled, pool, tab, tiles, ints([0] * n), ints(list(range(n))), 0, 0, H, Lk, Dk, 0.3, window)
+        results["prompt tiles on the matrix unit"] = tiled.float().cpu().view(n, H, Lk)
+        alone = torch.full_like(out, math.nan)
+        ops.attn_latent_mfma(qa, alone, pool, tab, None, ints([0] * n), ints(list(range(n))), 0, n, H, Lk, Dk, 0.3, window)
+        results["single tokens on the matrix unit"] = alone.float().cpu().view(n, H, Lk)
+    for how, got in results.items():
+        for p in range(n):
+            lo = max(0, p - window + 1)
+            want = torch.zeros(Lk)
+            for j in range(lo, p + 1):
+                want[j % Lk] += 1.0 / (p - lo + 1)
+            for h in range(H):
+                close(got[p, h], q(want, dt), dt, f"{how}: position {p} head {h}", bf16=2.0 ** -7)
 
 
 @pytest.mark.parametrize("dt", DTS)

@@ -193,6 +193,13 @@ int tm_rotate_heads(const void* src, int ld_src, int src_head, void* dst, int ld
 int tm_attn_latent(const void* qa, int q_stride, void* out, int out_stride, const void* pool, const int* block_tables,
                    int table_width, const int* seq_of_token, const int* positions, int T, int H, int Lk, int Dk, int page,
                    float scale, int window, int dtype, hipStream_t stream);
+// The same attention on the matrix unit (latent_mfma.hip), bfloat16: the prompt tiles of a step (tiles as for
+// tm_attn_prefill_mfma) or its single tokens (rows first_single .. first_single + n_single - 1), one of the two per call.
+int tm_attn_latent_mfma_takes(int Lk, int Dk, int q_stride, int out_stride);
+int tm_attn_latent_mfma(const void* qa, int q_stride, void* out, int out_stride, const void* pool, const int* block_tables,
+                        int table_width, const int* tiles, int n_tiles, const int* seq_of_token, const int* positions,
+                        int first_single, int n_single, int H, int Lk, int Dk, int page, float scale, int window,
+                        hipStream_t stream);
 
 // Experts chosen by a table row of the token id (moe.hip): see the head of that file.
 int tm_moe_route(const int* ids, const int* table, int T, int top, int E, int tile_rows, int* slot_pair, int* pair_slot,
@@ -203,6 +210,17 @@ int tm_moe_down(const void* act, const void* W, float* part, const int* tiles, c
                 int dtype, hipStream_t stream);
 int tm_moe_combine(const float* part, const int* pair_slot, void* y, int T, int top, float weight, int N, int dtype,
                    hipStream_t stream);
+
+// The per-head products and the experts' products on the matrix unit (grouped_mfma.hip), bfloat16; the matrices as
+// [groups, N, K] with k contiguous. The *_takes functions say whether the operands come in whole 16-byte pieces.
+int tm_heads_matmul_mfma_takes(const void* A, int lda, int a_off, const void* W, int K);
+int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const void* W, void* C, int ldc, int c_off, const float* gate, int ldg,
+                         int T, int H, int K, int N, hipStream_t stream);
+int tm_moe_mfma_takes(const void* x, int ldx, const void* Wgu, const void* Wd, const void* act, int K, int F);
+int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
+                        const int* n_tiles, int max_tiles, int K, int F, hipStream_t stream);
+int tm_moe_down_mfma(const void* act, const void* W, float* part, const int* tiles, const int* n_tiles, int max_tiles, int F, int N,
+                     hipStream_t stream);
 
 int tm_argmax_work_chunks(int V);
 int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);

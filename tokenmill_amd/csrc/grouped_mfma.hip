@@ -1,0 +1,158 @@
+// Products group by group on MFMA, bfloat16: C[row, n] = sum_k A[row, k] * W[group][n, k], every group with a matrix of its
+// own (W [groups, N, K], k contiguous). Two ways to say which rows belong to which group:
+//   heads   : every row has all groups; group h reads columns h * a_off .. + K of A and writes columns h * c_off .. + N of C
+//             (the per-head matrices of an attention); optionally times sigmoid(gate[row, h]);
+//   experts : tiles (group, first slot, rows <= 32) from tm_moe_route; a tile's rows are slots first .. first + rows - 1, and
+//             slot i reads row row_src[i] / src_div of A (row_src null: row i).
+// Epilogues: a plain store in bfloat16 or in 32-bit, or, with a matrix of 2 N rows (gate rows, then up rows),
+// silu(gate product) * up product. A block is RT tiles of 16 rows by 64 columns; its four wavefronts take 16 columns each;
+// k ascends in steps of 32 through LDS, so an element's sum has one order wherever its row stands.
+#include "common.h"
+#include "api.h"
+#include "attention_prefill_common.h"
+
+#define GM_BN 64
+#define GM_BK 32
+#define GM_LD (GM_BK + 8)
+
+enum { GM_STORE = 0, GM_STORE_F32 = 1, GM_SILU_MUL = 2 };
+
+template <int RT, int MODE>
+__global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restrict__ A, int lda, int a_off,
+                                                           const int* __restrict__ row_src, int src_div,
+                                                           const bf16_t* __restrict__ W, void* __restrict__ Cv, int ldc, int c_off,
+                                                           const float* __restrict__ gate, int ldg, const int* __restrict__ tiles,
+                                                           const int* __restrict__ n_tiles, int T, int K, int N) {
+    constexpr int BM = RT * 16;
+    constexpr bool GATED = MODE == GM_SILU_MUL;
+    __shared__ __align__(16) bf16_t As[BM][GM_LD];
+    __shared__ __align__(16) bf16_t Bs[GATED ? 2 : 1][GM_BN][GM_LD];
+    __shared__ int src[BM];
+    int group, row0, rows;
+    if (tiles) {
+        if ((int)blockIdx.x >= n_tiles[0]) return;
+        group = tiles[3 * blockIdx.x], row0 = tiles[3 * blockIdx.x + 1], rows = tiles[3 * blockIdx.x + 2];
+    } else {
+        group = blockIdx.z, row0 = blockIdx.x * BM, rows = min(BM, T - row0);
+    }
+    const int n0 = blockIdx.y * GM_BN;
+    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE, r = lane % 16, g = lane / 16;
+    const bf16_t* Wg = W + (size_t)group * (GATED ? 2 : 1) * N * K;
+    if (threadIdx.x < BM) {
+        const int i = threadIdx.x;
+        src[i] = i < rows ? (row_src ? row_src[row0 + i] / src_div : row0 + i) : -1;
+    }
+    __syncthreads();
+    f32x4_t acc[RT], acu[GATED ? RT : 1];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < (GATED ? RT : 1); ++t) acu[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += GM_BK) {
+        for (int idx = threadIdx.x; idx < BM * 4; idx += 256) {
+            const int i = idx / 4, c = idx % 4;
+            u32x4_t v = {0, 0, 0, 0};
+            if (src[i] >= 0 && k0 + 8 * c < K) v = *(const u32x4_t*)(A + (size_t)src[i] * lda + (size_t)group * a_off + k0 + 8 * c);
+            *(u32x4_t*)&As[i][8 * c] = v;
+        }
+        {
+            const int n = threadIdx.x / 4, c = threadIdx.x % 4;
+            const bool in = n0 + n < N && k0 + 8 * c < K;
+            u32x4_t v = {0, 0, 0, 0};
+            if (in) v = *(const u32x4_t*)(Wg + (size_t)(n0 + n) * K + k0 + 8 * c);
+            *(u32x4_t*)&Bs[0][n][8 * c] = v;
+            if (GATED) {
+                u32x4_t u = {0, 0, 0, 0};
+                if (in) u = *(const u32x4_t*)(Wg + (size_t)(N + n0 + n) * K + k0 + 8 * c);
+                *(u32x4_t*)&Bs[GATED ? 1 : 0][n][8 * c] = u;
+            }
+        }
+        __syncthreads();
+        PFrag bf, bu;
+        bf.u = *(const u32x4_t*)&Bs[0][16 * wave + r][8 * g];
+        if (GATED) bu.u = *(const u32x4_t*)&Bs[GATED ? 1 : 0][16 * wave + r][8 * g];
+#pragma unroll
+        for (int t = 0; t < RT; ++t) {
+            PFrag af;
+            af.u = *(const u32x4_t*)&As[16 * t + r][8 * g];
+            // rows of A as the first operand: the result holds C[row 4 g + i][column r]
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bf.b, acc[t], 0, 0, 0);
+            if (GATED) acu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bu.b, acu[t], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+    const int n = n0 + 16 * wave + r;
+    if (n >= N) return;
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = 16 * t + 4 * g + i;
+            if (row >= rows) continue;
+            const size_t at = (size_t)(row0 + row) * ldc + (size_t)group * c_off + n;
+            float v = acc[t][i];
+            if (MODE == GM_SILU_MUL) {
+                const float u = acu[t][i];
+                ((bf16_t*)Cv)[at] = f32_to_bf16(v / (1.0f + __expf(-v)) * u);
+            } else if (MODE == GM_STORE_F32) {
+                ((float*)Cv)[at] = v;
+            } else {
+                if (gate) v *= 1.0f / (1.0f + __expf(-gate[(size_t)(row0 + row) * ldg + group]));
+                ((bf16_t*)Cv)[at] = f32_to_bf16(v);
+            }
+        }
+}
+
+static bool gm_aligned(const void* p) { return ((uintptr_t)p % 16) == 0; }
+
+// Whether the per-head product takes these operands: K, the row strides of A and the heads' offsets in whole 16-byte pieces.
+extern "C" int tm_heads_matmul_mfma_takes(const void* A, int lda, int a_off, const void* W, int K) {
+    return gm_aligned(A) && gm_aligned(W) && K % 8 == 0 && lda % 8 == 0 && a_off % 8 == 0;
+}
+
+// C[t, h * c_off + n] = sum_k A[t, h * a_off + k] * W[h][n][k] (W [H, N, K]), times sigmoid(gate[t * ldg + h]) if gate.
+extern "C" int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const void* W, void* C, int ldc, int c_off, const float* gate,
+                                    int ldg, int T, int H, int K, int N, hipStream_t stream) {
+    if (!A || !W || !C || T < 0 || H <= 0 || H > 65535 || K <= 0 || N <= 0 || a_off < K || c_off < N ||
+        !tm_heads_matmul_mfma_takes(A, lda, a_off, W, K) || (gate && ldg < H))
+        return TM_ERR_ARG;
+    if (T == 0) return TM_OK;
+    dim3 grid((T + 63) / 64, (N + GM_BN - 1) / GM_BN, H);
+    if (grid.y > 65535) return TM_ERR_ARG;
+    grouped_mfma_kernel<4, GM_STORE><<<grid, 256, 0, stream>>>((const bf16_t*)A, lda, a_off, nullptr, 1, (const bf16_t*)W, C, ldc, c_off,
+                                                               gate, ldg, nullptr, nullptr, T, K, N);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// The experts' products of moe.hip on MFMA: the same operands, bfloat16, K and F multiples of 8, the route's tiles of 32 rows.
+extern "C" int tm_moe_mfma_takes(const void* x, int ldx, const void* Wgu, const void* Wd, const void* act, int K, int F) {
+    return gm_aligned(x) && gm_aligned(Wgu) && gm_aligned(Wd) && gm_aligned(act) && K % 8 == 0 && F % 8 == 0 && ldx % 8 == 0;
+}
+
+extern "C" int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
+                                   const int* n_tiles, int max_tiles, int K, int F, hipStream_t stream) {
+    if (!x || !slot_pair || !W || !act || !tiles || !n_tiles || top <= 0 || K <= 0 || F <= 0 || ldx < K || max_tiles < 0 || K % 8 ||
+        ldx % 8 || !gm_aligned(x) || !gm_aligned(W))
+        return TM_ERR_ARG;
+    if (max_tiles == 0) return TM_OK;
+    dim3 grid(max_tiles, (F + GM_BN - 1) / GM_BN);
+    if (grid.y > 65535) return TM_ERR_ARG;
+    grouped_mfma_kernel<2, GM_SILU_MUL><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, 0,
+                                                                  nullptr, 0, tiles, n_tiles, 0, K, F);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+extern "C" int tm_moe_down_mfma(const void* act, const void* W, float* part, const int* tiles, const int* n_tiles, int max_tiles, int F,
+                                int N, hipStream_t stream) {
+    if (!act || !W || !part || !tiles || !n_tiles || F <= 0 || N <= 0 || max_tiles < 0 || F % 8 || !gm_aligned(act) || !gm_aligned(W))
+        return TM_ERR_ARG;
+    if (max_tiles == 0) return TM_OK;
+    dim3 grid(max_tiles, (N + GM_BN - 1) / GM_BN);
+    if (grid.y > 65535) return TM_ERR_ARG;
+    grouped_mfma_kernel<2, GM_STORE_F32><<<grid, 256, 0, stream>>>((const bf16_t*)act, F, 0, nullptr, 1, (const bf16_t*)W, part, N, 0,
+                                                                   nullptr, 0, tiles, n_tiles, 0, F, N);
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}

@@ -1479,6 +1479,42 @@ def attn_latent(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, block_t
     return out
 
 
+def attn_latent_mfma_takes(dtype, Lk: int, Dk: int, H: int) -> bool:
+    """Does the matrix-unit kernel run these sizes (bfloat16, latent and row in whole 16-byte pieces)?"""
+    return dtype == torch.bfloat16 and bool(library().tm_attn_latent_mfma_takes(c_int(Lk), c_int(Dk), c_int(H * Dk), c_int(H * Lk)))
+
+
+def attn_latent_mfma(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, block_tables: torch.Tensor, tiles: torch.Tensor | None,
+                     seq_of_token: torch.Tensor, positions: torch.Tensor, first_single: int, n_single: int, H: int, Lk: int, Dk: int,
+                     scale: float, window: int = 0) -> torch.Tensor:
+    """``attn_latent`` on the matrix unit for bfloat16: with ``tiles`` (int32 [n, 4]: request, first row, tokens, first position)
+    the prompt portions of the step, tile by tile; with ``tiles`` None the ``n_single`` single tokens that start at row
+    ``first_single``. Rows of qa / out that neither names are left alone."""
+    _gpu(qa, out, pool, block_tables, tiles, seq_of_token, positions)
+    T = qa.shape[0]
+    _need(qa.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "attention(latent, matrix unit): bfloat16 only")
+    _need(qa.is_contiguous() and tuple(qa.shape) == (T, H * Dk) and out.is_contiguous() and tuple(out.shape) == (T, H * Lk),
+          f"attention(latent, matrix unit): qa [T, {H * Dk}] and out [T, {H * Lk}] contiguous")
+    _need(attn_latent_mfma_takes(qa.dtype, Lk, Dk, H), "attention(latent, matrix unit): sizes the kernel does not run")
+    page = _check_latent_pool(pool, Dk, qa.dtype, "attention(latent, matrix unit)")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "attention(latent, matrix unit): block_tables must be contiguous int32 [S, W]")
+    _ints(seq_of_token, T, "seq_of_token")
+    _ints(positions, T, "positions")
+    n_tiles = 0
+    if tiles is not None:
+        _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(), "tiles must be int32 [n, 4]")
+        n_tiles, n_single = tiles.shape[0], 0
+    else:
+        _need(0 <= first_single and first_single + n_single <= T, "attention(latent, matrix unit): the single tokens lie outside the step")
+    _need(window >= 0, "attention(latent, matrix unit): window must be >= 0")
+    _check(library().tm_attn_latent_mfma(_p(qa), c_int(H * Dk), _p(out), c_int(H * Lk), _p(pool), _p(block_tables),
+                                         c_int(block_tables.shape[1]), _p(tiles), c_int(n_tiles), _p(seq_of_token), _p(positions),
+                                         c_int(first_single), c_int(n_single), c_int(H), c_int(Lk), c_int(Dk), c_int(page),
+                                         c_float(scale), c_int(window), _stream()), "attn_latent_mfma")
+    return out
+
+
 # -------------------------------------------------------------------------------------------- experts by table
 
 MOE_TILE_ROWS = 32

@@ -114,6 +114,22 @@ class LatentAttention(Mixer):
         seen, pairs = self.visible_pairs(step)
         return seen * self.row * e + step.num_tokens * H * (self.row + Lk) * e, 2 * pairs * H * (self.row + Lk)
 
+    def _attend(self, qa, latent, step: StepContext, cache: KVCacheView, group) -> None:
+        """Prompt portions and single tokens (the step's last ``num_decode`` rows) on the matrix unit where its kernel takes
+        the sizes; the 32-bit path and every other size through the kernel that takes a token and a head a wavefront."""
+        H, Lk, row, T = self.num_heads, self.kv_rank, self.row, qa.shape[0]
+        tiles, first_single = step.prefill_tiles, T - step.num_decode
+        if not ops.attn_latent_mfma_takes(qa.dtype, Lk, row, H) or (first_single > 0 and (tiles is None or not tiles.shape[0])):
+            ops.attn_latent(qa, latent, cache.k, group.block_tables, step.seq_of_token, step.positions, H, Lk, row, self.scale,
+                            self.window or 0)
+            return
+        if first_single > 0:
+            ops.attn_latent_mfma(qa, latent, cache.k, group.block_tables, tiles, step.seq_of_token, step.positions, 0, 0, H, Lk, row,
+                                 self.scale, self.window or 0)
+        if step.num_decode > 0:
+            ops.attn_latent_mfma(qa, latent, cache.k, group.block_tables, None, step.seq_of_token, step.positions, first_single,
+                                 step.num_decode, H, Lk, row, self.scale, self.window or 0)
+
     def forward(self, x, step: StepContext, cache: KVCacheView, residual: torch.Tensor | None = None):
         x = as_tensor(x)
         T = x.shape[0]
@@ -135,8 +151,7 @@ class LatentAttention(Mixer):
                 ops.rotate_heads(q[:, Dn:], Dn + Dr, qa[:, Lk:], row, H, Dr, cos, sin, step.positions)
         latent = torch.empty((T, H * Lk), dtype=x.dtype, device=x.device)
         with profiling.label("attention", lambda: self.cost("attention", step, T)):
-            ops.attn_latent(qa, latent, cache.k, group.block_tables, step.seq_of_token, step.positions, H, Lk, row, self.scale,
-                            self.window or 0)
+            self._attend(qa, latent, step, cache, group)
         with profiling.label("o_proj", lambda: self.cost("o_proj", step, T)):
             out = torch.empty((T, H * Dv), dtype=x.dtype, device=x.device)
             ops.heads_matmul(latent, Lk, self.uv, out, Dv, gate=low[:, Lq + row:] if self.output_gate else None)
