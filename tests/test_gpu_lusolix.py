@@ -127,11 +127,11 @@ def test_poly_norm(dt, F):
 
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("T,H,K,N", [(1, 3, 20, 36), (37, 2, 72, 8), (130, 5, 8, 100), (4, 1, 44, 40)])
+@pytest.mark.parametrize("T,H,K,N", [(1, 3, 20, 36), (37, 2, 72, 8), (130, 5, 8, 100), (4, 1, 44, 40), (200, 3, 64, 96)])
 def test_products_head_by_head(dt, T, H, K, N):
     from tokenmill_amd.hip import ops
     torch.manual_seed(T + H)
-    pad_a, pad_c = 6, 4
+    pad_a, pad_c = (6, 4) if K % 8 else (8, 4)
     a = q(torch.randn(T, H * (K + pad_a)), dt)
     b = q(torch.randn(H, K, N) * 0.3, dt)
     gate = torch.randn(T, H + 3)
@@ -141,6 +141,18 @@ def test_products_head_by_head(dt, T, H, K, N):
     got = c.float().cpu().view(T, H, N + pad_c)
     close(got[..., :N], q(want, dt), dt, "per-head product")
     assert bool((got[..., N:] == 7.0).all()), "wrote beyond a head's columns"
+    if dt == torch.bfloat16 and K % 8 == 0:
+        # the matrix unit, from the matrices as [H, N, K]; a row alone gives the bits it has among the others
+        ad, wd = a.to(dt).to(DEV), b.transpose(1, 2).contiguous().to(dt).to(DEV)
+        assert ops.heads_matmul_mfma_takes(ad, K + pad_a, wd)
+        c2 = torch.full((T, H * (N + pad_c)), 7.0, dtype=dt, device=DEV)
+        ops.heads_matmul_mfma(ad, K + pad_a, wd, c2, N + pad_c, gate=gate.to(DEV)[:, 2:])
+        got2 = c2.float().cpu().view(T, H, N + pad_c)
+        close(got2[..., :N], q(want, dt), dt, "per-head product on the matrix unit")
+        assert bool((got2[..., N:] == 7.0).all()), "wrote beyond a head's columns"
+        one = torch.zeros((1, H * (N + pad_c)), dtype=dt, device=DEV)
+        ops.heads_matmul_mfma(ad[T // 2:T // 2 + 1], K + pad_a, wd, one, N + pad_c, gate=gate.to(DEV)[T // 2:T // 2 + 1, 2:])
+        assert torch.equal(one.float().cpu().view(H, N + pad_c)[:, :N], got2[T // 2, :, :N])
 
 
 def _experts_fixture(dt, width, ff, experts, top, vocab, seed):
@@ -158,7 +170,8 @@ def _experts_fixture(dt, width, ff, experts, top, vocab, seed):
 
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("width,ff,experts,top,T", [(96, 40, 5, 2, 77), (80, 16, 3, 3, 9), (80, 52, 4, 1, 1), (72, 32, 9, 2, 200), (64, 24, 40, 4, 3)])
+@pytest.mark.parametrize("width,ff,experts,top,T", [(96, 40, 5, 2, 77), (80, 16, 3, 3, 9), (80, 52, 4, 1, 1), (72, 32, 9, 2, 200), (64, 24, 40, 4, 3),
+                                                      (96, 40, 5, 2, 300), (80, 16, 3, 3, 60)])
 def test_experts_by_table(dt, width, ff, experts, top, T):
     from types import SimpleNamespace
     vocab = 50
@@ -286,7 +299,7 @@ def test_rows_just_inside_and_just_outside_the_window_show(dt, window, page):
         ops.attn_latent_mfma(qa, tiled, pool, tab, tiles, ints([0] * n), ints(list(range(n))), 0, 0, H, Lk, Dk, 0.3, window)
         results["prompt tiles on the matrix unit"] = tiled.float().cpu().view(n, H, Lk)
         alone = torch.full_like(out, math.nan)
-        ops.attn_latent_mfma(qa, alone, pool, tab, None, ints([0] * n), ints(list(range(n))), 0, n, H, Lk, Dk, 0.3, window)
+        ops.attn_latent_mfma(qa, alone, pool, tab, None, ints([0] * n), ints(list(range(n))), 0, n, H, Lk, Dk, 0.3, window, most_context=n)
         results["single tokens on the matrix unit"] = alone.float().cpu().view(n, H, Lk)
     for how, got in results.items():
         for p in range(n):
@@ -322,6 +335,19 @@ def test_one_far_row_among_hundreds_dominates(dt):
     got = out.float().cpu().view(2, H, Lk)
     close(got[0, 1], rows[13, :Lk], dt, "row 13 is the window's last for position 598", bf16=2.0 ** -6)
     assert float((got[1, 1] - rows[13, :Lk]).abs().max()) > 0.05, "row 13 is outside the window of position 599"
+    if dt == torch.bfloat16:
+        # the matrix unit: the two tokens alone (their rows in chunks over several blocks, merged), then as a prompt tile
+        tile = torch.tensor([[0, 0, 2, 598]], dtype=torch.int32, device=DEV)
+        for tiles, window in ((None, 0), (None, 586), (tile, 0), (tile, 586)):
+            out.fill_(math.nan)
+            ops.attn_latent_mfma(qa, out, pool, table, tiles, ints([0, 0]), ints([598, 599]), 0, 2, H, Lk, Dk, 1.0, window, most_context=600)
+            got = out.float().cpu().view(2, H, Lk)
+            close(got[0, 1], rows[13, :Lk], dt, "the far row, matrix unit", bf16=2.0 ** -6)
+            if window:
+                assert float((got[1, 1] - rows[13, :Lk]).abs().max()) > 0.05, "row 13 is outside the window of position 599"
+            else:
+                close(got[1, 1], rows[13, :Lk], dt, "the far row, matrix unit", bf16=2.0 ** -6)
+                close(got[1, 0], q(rows[:600, :Lk].mean(0), dt), dt, "the mean, matrix unit", bf16=2.0 ** -4)
 
 
 # ----------------------------------------------------------------------------------------------- whole models

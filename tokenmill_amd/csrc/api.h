@@ -196,10 +196,15 @@ int tm_attn_latent(const void* qa, int q_stride, void* out, int out_stride, cons
 // The same attention on the matrix unit (latent_mfma.hip), bfloat16: the prompt tiles of a step (tiles as for
 // tm_attn_prefill_mfma) or its single tokens (rows first_single .. first_single + n_single - 1), one of the two per call.
 int tm_attn_latent_mfma_takes(int Lk, int Dk, int q_stride, int out_stride);
+// Single tokens have their visible rows dealt in chunks of chunk_runs = tm_attn_latent_chunk_runs(the most rows the model lets
+// a token see) runs to blocks of their own: tm_attn_latent_chunks(most rows a token of the call sees, chunk_runs) chunks,
+// part_o [n_single * H, chunks, Lk] and part_ml [n_single * H, chunks, 2] 32-bit scratch.
+int tm_attn_latent_chunk_runs(int bound);
+int tm_attn_latent_chunks(int most_rows, int chunk_runs);
 int tm_attn_latent_mfma(const void* qa, int q_stride, void* out, int out_stride, const void* pool, const int* block_tables,
                         int table_width, const int* tiles, int n_tiles, const int* seq_of_token, const int* positions,
-                        int first_single, int n_single, int H, int Lk, int Dk, int page, float scale, int window,
-                        hipStream_t stream);
+                        int first_single, int n_single, float* part_o, float* part_ml, int n_chunks, int chunk_runs, int H, int Lk,
+                        int Dk, int page, float scale, int window, hipStream_t stream);
 
 // Experts chosen by a table row of the token id (moe.hip): see the head of that file.
 int tm_moe_route(const int* ids, const int* table, int T, int top, int E, int tile_rows, int* slot_pair, int* pair_slot,
@@ -218,9 +223,9 @@ int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const void* W, void*
                          int T, int H, int K, int N, hipStream_t stream);
 int tm_moe_mfma_takes(const void* x, int ldx, const void* Wgu, const void* Wd, const void* act, int K, int F);
 int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
-                        const int* n_tiles, int max_tiles, int K, int F, hipStream_t stream);
-int tm_moe_down_mfma(const void* act, const void* W, float* part, const int* tiles, const int* n_tiles, int max_tiles, int F, int N,
-                     hipStream_t stream);
+                        const int* n_tiles, int max_tiles, int tile_rows, int K, int F, hipStream_t stream);
+int tm_moe_down_mfma(const void* act, const void* W, float* part, const int* tiles, const int* n_tiles, int max_tiles, int tile_rows,
+                     int F, int N, hipStream_t stream);
 
 int tm_argmax_work_chunks(int V);
 int tm_argmax_rows(const float* logits, int R, int V, int* out, float* work_v, int* work_i, hipStream_t stream);

@@ -48,26 +48,38 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
     for (int t = 0; t < RT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < (GATED ? RT : 1); ++t) acu[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    // a thread's pieces of a k-step: RT / 4 of A (one if RT = 2 and the thread is among the first 128), one of W (two with
+    // a gate); those of the step after the current one are asked for before the current one is multiplied
+    constexpr int NA = (BM * 4 + 255) / 256;
+    u32x4_t ha[NA], hb, hu;
+    const int bn = threadIdx.x / 4, bc = threadIdx.x % 4;
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int u = 0; u < NA; ++u) {
+            const int idx = threadIdx.x + 256 * u, i = idx / 4, c = idx % 4;
+            ha[u] = u32x4_t{0, 0, 0, 0};
+            if (idx < BM * 4 && src[i] >= 0 && k0 + 8 * c < K)
+                ha[u] = *(const u32x4_t*)(A + (size_t)src[i] * lda + (size_t)group * a_off + k0 + 8 * c);
+        }
+        const bool in = n0 + bn < N && k0 + 8 * bc < K;
+        hb = u32x4_t{0, 0, 0, 0};
+        if (in) hb = *(const u32x4_t*)(Wg + (size_t)(n0 + bn) * K + k0 + 8 * bc);
+        if (GATED) {
+            hu = u32x4_t{0, 0, 0, 0};
+            if (in) hu = *(const u32x4_t*)(Wg + (size_t)(N + n0 + bn) * K + k0 + 8 * bc);
+        }
+    };
+    fetch(0);
     for (int k0 = 0; k0 < K; k0 += GM_BK) {
-        for (int idx = threadIdx.x; idx < BM * 4; idx += 256) {
-            const int i = idx / 4, c = idx % 4;
-            u32x4_t v = {0, 0, 0, 0};
-            if (src[i] >= 0 && k0 + 8 * c < K) v = *(const u32x4_t*)(A + (size_t)src[i] * lda + (size_t)group * a_off + k0 + 8 * c);
-            *(u32x4_t*)&As[i][8 * c] = v;
+#pragma unroll
+        for (int u = 0; u < NA; ++u) {
+            const int idx = threadIdx.x + 256 * u;
+            if (idx < BM * 4) *(u32x4_t*)&As[idx / 4][8 * (idx % 4)] = ha[u];
         }
-        {
-            const int n = threadIdx.x / 4, c = threadIdx.x % 4;
-            const bool in = n0 + n < N && k0 + 8 * c < K;
-            u32x4_t v = {0, 0, 0, 0};
-            if (in) v = *(const u32x4_t*)(Wg + (size_t)(n0 + n) * K + k0 + 8 * c);
-            *(u32x4_t*)&Bs[0][n][8 * c] = v;
-            if (GATED) {
-                u32x4_t u = {0, 0, 0, 0};
-                if (in) u = *(const u32x4_t*)(Wg + (size_t)(N + n0 + n) * K + k0 + 8 * c);
-                *(u32x4_t*)&Bs[GATED ? 1 : 0][n][8 * c] = u;
-            }
-        }
+        *(u32x4_t*)&Bs[0][bn][8 * bc] = hb;
+        if (GATED) *(u32x4_t*)&Bs[GATED ? 1 : 0][bn][8 * bc] = hu;
         __syncthreads();
+        if (k0 + GM_BK < K) fetch(k0 + GM_BK);
         PFrag bf, bu;
         bf.u = *(const u32x4_t*)&Bs[0][16 * wave + r][8 * g];
         if (GATED) bu.u = *(const u32x4_t*)&Bs[GATED ? 1 : 0][16 * wave + r][8 * g];
@@ -125,34 +137,43 @@ extern "C" int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const voi
     return TM_OK;
 }
 
-// The experts' products of moe.hip on MFMA: the same operands, bfloat16, K and F multiples of 8, the route's tiles of 32 rows.
+// The experts' products of moe.hip on MFMA: the same operands, bfloat16, K and F multiples of 8, the route's tiles of
+// tile_rows = 32, 64 or 128 rows (the larger, the fewer times an expert's matrices are read).
 extern "C" int tm_moe_mfma_takes(const void* x, int ldx, const void* Wgu, const void* Wd, const void* act, int K, int F) {
     return gm_aligned(x) && gm_aligned(Wgu) && gm_aligned(Wd) && gm_aligned(act) && K % 8 == 0 && F % 8 == 0 && ldx % 8 == 0;
 }
 
 extern "C" int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
-                                   const int* n_tiles, int max_tiles, int K, int F, hipStream_t stream) {
+                                   const int* n_tiles, int max_tiles, int tile_rows, int K, int F, hipStream_t stream) {
+    if (tile_rows != 32 && tile_rows != 64 && tile_rows != 128) return TM_ERR_ARG;
     if (!x || !slot_pair || !W || !act || !tiles || !n_tiles || top <= 0 || K <= 0 || F <= 0 || ldx < K || max_tiles < 0 || K % 8 ||
         ldx % 8 || !gm_aligned(x) || !gm_aligned(W))
         return TM_ERR_ARG;
     if (max_tiles == 0) return TM_OK;
     dim3 grid(max_tiles, (F + GM_BN - 1) / GM_BN);
     if (grid.y > 65535) return TM_ERR_ARG;
-    grouped_mfma_kernel<2, GM_SILU_MUL><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, 0,
-                                                                  nullptr, 0, tiles, n_tiles, 0, K, F);
+#define GM_GO(RT_)                                                                                                             \
+    grouped_mfma_kernel<RT_, GM_SILU_MUL><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
+                                                                    0, nullptr, 0, tiles, n_tiles, 0, K, F)
+    if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
+#undef GM_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
 
-extern "C" int tm_moe_down_mfma(const void* act, const void* W, float* part, const int* tiles, const int* n_tiles, int max_tiles, int F,
-                                int N, hipStream_t stream) {
+extern "C" int tm_moe_down_mfma(const void* act, const void* W, float* part, const int* tiles, const int* n_tiles, int max_tiles,
+                                int tile_rows, int F, int N, hipStream_t stream) {
+    if (tile_rows != 32 && tile_rows != 64 && tile_rows != 128) return TM_ERR_ARG;
     if (!act || !W || !part || !tiles || !n_tiles || F <= 0 || N <= 0 || max_tiles < 0 || F % 8 || !gm_aligned(act) || !gm_aligned(W))
         return TM_ERR_ARG;
     if (max_tiles == 0) return TM_OK;
     dim3 grid(max_tiles, (N + GM_BN - 1) / GM_BN);
     if (grid.y > 65535) return TM_ERR_ARG;
-    grouped_mfma_kernel<2, GM_STORE_F32><<<grid, 256, 0, stream>>>((const bf16_t*)act, F, 0, nullptr, 1, (const bf16_t*)W, part, N, 0,
-                                                                   nullptr, 0, tiles, n_tiles, 0, F, N);
+#define GM_GO(RT_)                                                                                                              \
+    grouped_mfma_kernel<RT_, GM_STORE_F32><<<grid, 256, 0, stream>>>((const bf16_t*)act, F, 0, nullptr, 1, (const bf16_t*)W, part, N, 0, \
+                                                                     nullptr, 0, tiles, n_tiles, 0, F, N)
+    if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
+#undef GM_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

@@ -1435,6 +1435,39 @@ def heads_matmul(a: torch.Tensor, a_head: int, b: torch.Tensor, c: torch.Tensor,
     return c
 
 
+def heads_matmul_mfma_takes(a: torch.Tensor, a_head: int, w: torch.Tensor) -> bool:
+    """Does the matrix-unit kernel take this per-head product (bfloat16, whole 16-byte pieces)? w [H, N, K]."""
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or not a.is_cuda:
+        return False
+    lda = a.stride(0) if a.shape[0] > 1 else max(a.stride(0), a.shape[1])
+    return bool(library().tm_heads_matmul_mfma_takes(_p(a), c_int(lda), c_int(a_head), _p(w), c_int(w.shape[2])))
+
+
+def heads_matmul_mfma(a: torch.Tensor, a_head: int, w: torch.Tensor, c: torch.Tensor, c_head: int,
+                      gate: torch.Tensor | None = None) -> torch.Tensor:
+    """``heads_matmul`` on the matrix unit, with the matrices given as w [H, N, K] (k contiguous): c[t, h * c_head + n] =
+    sum_k a[t, h * a_head + k] * w[h, n, k], times sigmoid(gate[t, h]) if ``gate`` (float32 [T, >= H])."""
+    _gpu(a, w, c, gate)
+    T = a.shape[0]
+    H, N, K = w.shape
+    _need(a.dim() == 2 and c.dim() == 2 and a.stride(1) == 1 and c.stride(1) == 1 and c.shape[0] == T and w.is_contiguous(),
+          "heads_matmul: a, c [T, .] with unit inner stride, w contiguous [H, N, K]")
+    _need(a.dtype == w.dtype == c.dtype == torch.bfloat16, "heads_matmul (matrix unit): bfloat16")
+    _need(a_head >= K and c_head >= N and a.shape[1] >= (H - 1) * a_head + K and c.shape[1] >= (H - 1) * c_head + N,
+          "heads_matmul: the heads do not fit the rows")
+    _need(heads_matmul_mfma_takes(a, a_head, w), "heads_matmul (matrix unit): operands not in whole 16-byte pieces")
+    gate_stride = 0
+    if gate is not None:
+        _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= H and gate.stride(1) == 1,
+              "heads_matmul: gate is float32 [T, >= H]")
+        gate_stride = gate.stride(0) if T > 1 else max(gate.stride(0), H)
+    lda = a.stride(0) if T > 1 else max(a.stride(0), a.shape[1])
+    ldc = c.stride(0) if T > 1 else max(c.stride(0), c.shape[1])
+    _check(library().tm_heads_matmul_mfma(_p(a), c_int(lda), c_int(a_head), _p(w), _p(c), c_int(ldc), c_int(c_head), _p(gate),
+                                          c_int(gate_stride), c_int(T), c_int(H), c_int(K), c_int(N), _stream()), "heads_matmul_mfma")
+    return c
+
+
 def rotate_heads(src: torch.Tensor, src_head: int, dst: torch.Tensor, dst_head: int, H: int, Dr: int, cos: torch.Tensor | None,
                  sin: torch.Tensor | None, positions: torch.Tensor | None) -> None:
     """dst[t, h * dst_head + c] = src[t, h * src_head + c] for c < Dr, the first 2 * cos.shape[1] channels of every head rotated in
@@ -1486,10 +1519,12 @@ def attn_latent_mfma_takes(dtype, Lk: int, Dk: int, H: int) -> bool:
 
 def attn_latent_mfma(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, block_tables: torch.Tensor, tiles: torch.Tensor | None,
                      seq_of_token: torch.Tensor, positions: torch.Tensor, first_single: int, n_single: int, H: int, Lk: int, Dk: int,
-                     scale: float, window: int = 0) -> torch.Tensor:
+                     scale: float, window: int = 0, most_context: int = 0, bound: int = 0) -> torch.Tensor:
     """``attn_latent`` on the matrix unit for bfloat16: with ``tiles`` (int32 [n, 4]: request, first row, tokens, first position)
     the prompt portions of the step, tile by tile; with ``tiles`` None the ``n_single`` single tokens that start at row
-    ``first_single``. Rows of qa / out that neither names are left alone."""
+    ``first_single``, none of which sits beyond position ``most_context`` - 1 (their visible rows are dealt in chunks to blocks
+    of their own and merged in chunk order; ``bound``: the most rows the model lets any token see, its window or its longest
+    context, which sets the chunks' size). Rows of qa / out that neither names are left alone."""
     _gpu(qa, out, pool, block_tables, tiles, seq_of_token, positions)
     T = qa.shape[0]
     _need(qa.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "attention(latent, matrix unit): bfloat16 only")
@@ -1501,17 +1536,22 @@ def attn_latent_mfma(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, bl
           "attention(latent, matrix unit): block_tables must be contiguous int32 [S, W]")
     _ints(seq_of_token, T, "seq_of_token")
     _ints(positions, T, "positions")
-    n_tiles = 0
+    _need(window >= 0, "attention(latent, matrix unit): window must be >= 0")
+    n_tiles, n_chunks, chunk_runs, part_o, part_ml = 0, 0, 0, None, None
     if tiles is not None:
         _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(), "tiles must be int32 [n, 4]")
         n_tiles, n_single = tiles.shape[0], 0
-    else:
+    elif n_single > 0:
         _need(0 <= first_single and first_single + n_single <= T, "attention(latent, matrix unit): the single tokens lie outside the step")
-    _need(window >= 0, "attention(latent, matrix unit): window must be >= 0")
+        _need(most_context > 0, "attention(latent, matrix unit): single tokens need the longest context among them")
+        chunk_runs = int(library().tm_attn_latent_chunk_runs(c_int(window if window else max(bound, most_context))))
+        n_chunks = int(library().tm_attn_latent_chunks(c_int(min(window, most_context) if window else most_context), c_int(chunk_runs)))
+        part_o = torch.empty((n_single * H, n_chunks, Lk), dtype=torch.float32, device=qa.device)
+        part_ml = torch.empty((n_single * H, n_chunks, 2), dtype=torch.float32, device=qa.device)
     _check(library().tm_attn_latent_mfma(_p(qa), c_int(H * Dk), _p(out), c_int(H * Lk), _p(pool), _p(block_tables),
                                          c_int(block_tables.shape[1]), _p(tiles), c_int(n_tiles), _p(seq_of_token), _p(positions),
-                                         c_int(first_single), c_int(n_single), c_int(H), c_int(Lk), c_int(Dk), c_int(page),
-                                         c_float(scale), c_int(window), _stream()), "attn_latent_mfma")
+                                         c_int(first_single), c_int(n_single), _p(part_o), _p(part_ml), c_int(n_chunks), c_int(chunk_runs), c_int(H),
+                                         c_int(Lk), c_int(Dk), c_int(page), c_float(scale), c_int(window), _stream()), "attn_latent_mfma")
     return out
 
 
@@ -1521,14 +1561,23 @@ MOE_TILE_ROWS = 32
 MOE_MAX_EXPERTS = 1024
 
 
-def moe_max_tiles(pairs: int, experts: int) -> int:
-    """The most tiles of MOE_TILE_ROWS rows that ``pairs`` (token, expert) pairs can fall into."""
-    return min(pairs, pairs // MOE_TILE_ROWS + experts)
+def moe_max_tiles(pairs: int, experts: int, tile_rows: int = MOE_TILE_ROWS) -> int:
+    """The most tiles of ``tile_rows`` rows that ``pairs`` (token, expert) pairs can fall into."""
+    return min(pairs, pairs // tile_rows + experts)
 
 
-def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int):
+def moe_tile_rows(pairs: int, experts: int, dtype) -> int:
+    """Rows of a tile for a step of ``pairs`` pairs: 32, or 64 / 128 where the matrix-unit products (bfloat16) have that many
+    rows an expert on average, so that an expert's matrices are read fewer times. A row's result does not depend on it."""
+    if dtype != torch.bfloat16:
+        return MOE_TILE_ROWS
+    per_expert = pairs // max(experts, 1)
+    return 128 if per_expert >= 96 else (64 if per_expert >= 48 else MOE_TILE_ROWS)
+
+
+def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS):
     """Sorts the step's (token, choice) pairs by expert. Returns int32 tensors (slot_pair [P], pair_slot [P], tiles [max, 3],
-    n_tiles [1]); see ``csrc/moe.hip``."""
+    n_tiles [1]) and the tiles' rows; see ``csrc/moe.hip``."""
     _gpu(token_ids, table)
     T = token_ids.numel()
     _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "moe_route: table is contiguous int32 [vocab, top]")
@@ -1536,19 +1585,20 @@ def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int):
     top = table.shape[1]
     _need(0 < experts <= MOE_MAX_EXPERTS, f"moe_route: up to {MOE_MAX_EXPERTS} experts")
     P = T * top
-    most = moe_max_tiles(P, experts)
+    _need(tile_rows in (32, 64, 128), "moe_route: tiles of 32, 64 or 128 rows")
+    most = moe_max_tiles(P, experts, tile_rows)
     work = torch.empty(2 * P + 3 * most + 1, dtype=torch.int32, device=token_ids.device)
     slot_pair, pair_slot, tiles, n_tiles = work[:P], work[P:2 * P], work[2 * P:2 * P + 3 * most].view(most, 3), work[2 * P + 3 * most:]
-    _check(library().tm_moe_route(_p(token_ids), _p(table), c_int(T), c_int(top), c_int(experts), c_int(MOE_TILE_ROWS), _p(slot_pair),
+    _check(library().tm_moe_route(_p(token_ids), _p(table), c_int(T), c_int(top), c_int(experts), c_int(tile_rows), _p(slot_pair),
                                   _p(pair_slot), _p(tiles), _p(n_tiles), _stream()), "moe_route")
-    return slot_pair, pair_slot, tiles, n_tiles
+    return slot_pair, pair_slot, tiles, n_tiles, tile_rows
 
 
 def moe_experts(x: torch.Tensor, routed, w_gate_up: torch.Tensor, w_down: torch.Tensor, top: int, weight: float,
                 out: torch.Tensor) -> torch.Tensor:
     """out[t] = sum over the token's ``top`` experts e of weight * Wd[e] (silu(Wg[e] x[t]) * (Wu[e] x[t])), in the order of
     its choices. w_gate_up [E, 2F, K] (gate rows, then up rows), w_down [E, N, F]; ``routed`` from ``moe_route``."""
-    slot_pair, pair_slot, tiles, n_tiles = routed
+    slot_pair, pair_slot, tiles, n_tiles, tile_rows = routed
     _gpu(x, w_gate_up, w_down, out)
     T, K = x.shape
     E, F2, K2 = w_gate_up.shape
@@ -1565,6 +1615,16 @@ def moe_experts(x: torch.Tensor, routed, w_gate_up: torch.Tensor, w_down: torch.
     part = torch.empty((P, N), dtype=torch.float32, device=x.device)
     lib, dt = library(), c_int(code(x.dtype))
     ldx = x.stride(0) if T > 1 else max(x.stride(0), K)
+    if x.dtype == torch.bfloat16 and lib.tm_moe_mfma_takes(_p(x), c_int(ldx), _p(w_gate_up), _p(w_down), _p(act), c_int(K), c_int(F)):
+        # the matrix unit takes the same tiles
+        _check(lib.tm_moe_gate_up_mfma(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_gate_up), _p(act), _p(tiles), _p(n_tiles),
+                                       c_int(most), c_int(tile_rows), c_int(K), c_int(F), _stream()), "moe_gate_up_mfma")
+        _check(lib.tm_moe_down_mfma(_p(act), _p(w_down), _p(part), _p(tiles), _p(n_tiles), c_int(most), c_int(tile_rows), c_int(F),
+                                    c_int(N), _stream()), "moe_down_mfma")
+        _check(lib.tm_moe_combine(_p(part), _p(pair_slot), _p(out), c_int(T), c_int(top), c_float(weight), c_int(N), dt, _stream()),
+               "moe_combine")
+        return out
+    _need(tile_rows == MOE_TILE_ROWS, "moe_experts: these products take tiles of 32 rows")
     _check(lib.tm_moe_gate_up(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_gate_up), _p(act), _p(tiles), _p(n_tiles), c_int(most),
                               c_int(K), c_int(F), dt, _stream()), "moe_gate_up")
     _check(lib.tm_moe_down(_p(act), _p(w_down), _p(part), _p(tiles), _p(n_tiles), c_int(most), c_int(F), c_int(N), dt, _stream()),

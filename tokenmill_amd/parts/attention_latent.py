@@ -60,6 +60,8 @@ class LatentAttention(Mixer):
         self.kv_norm: torch.Tensor | None = None
         self.uk: torch.Tensor | None = None             # [H, Dn, Lk]: a head's query channels onto the latent
         self.uv: torch.Tensor | None = None             # [H, Lk, Dv]: the latent onto a head's value channels
+        self.uk_nt: torch.Tensor | None = None          # the same two as [H, N, K], the order the matrix-unit products read
+        self.uv_nt: torch.Tensor | None = None
 
     def tensor_specs(self, prefix: str):
         H, Dn, Dv, Lk = self.num_heads, self.head_dim, self.v_head_dim, self.kv_rank
@@ -78,12 +80,18 @@ class LatentAttention(Mixer):
         self.uq.load(tensors, prefix)
         self.o.load(tensors, prefix)
         self.uk = tensors[prefix + self.names["uk"] + sw].view(H, Dn, Lk).contiguous()
-        self.uv = tensors[prefix + self.names["uv"] + sw].view(H, Dv, Lk).transpose(1, 2).contiguous()
+        self.uv_nt = tensors[prefix + self.names["uv"] + sw].view(H, Dv, Lk)
+        self.uv = self.uv_nt.transpose(1, 2).contiguous()
+        self.uk_nt = self.uk.transpose(1, 2).contiguous() if self.uk.dtype == torch.bfloat16 else None
         # the norm weights meet 32-bit statistics and are kept in 32-bit
         self.q_norm = tensors[prefix + self.norm_names[0]].float().contiguous()
         self.kv_norm = tensors[prefix + self.norm_names[1]].float().contiguous()
         if self.rotary is not None:
             self.rotary.load(tensors, prefix)
+
+    def prepare(self, pack_weights: bool) -> None:
+        for lin in (self.down, self.uq, self.o):
+            lin.prepare(pack_weights)
 
     def cache_spec(self):
         return KVCacheSpec(1, self.row, self.window, values=False)
@@ -128,7 +136,8 @@ class LatentAttention(Mixer):
                                  self.scale, self.window or 0)
         if step.num_decode > 0:
             ops.attn_latent_mfma(qa, latent, cache.k, group.block_tables, None, step.seq_of_token, step.positions, first_single,
-                                 step.num_decode, H, Lk, row, self.scale, self.window or 0)
+                                 step.num_decode, H, Lk, row, self.scale, self.window or 0, most_context=step.max_decode_context,
+                                 bound=self.rotary.max_positions if self.rotary is not None else 1 << 20)
 
     def forward(self, x, step: StepContext, cache: KVCacheView, residual: torch.Tensor | None = None):
         x = as_tensor(x)
@@ -146,7 +155,10 @@ class LatentAttention(Mixer):
                                group.slot_mapping if cache.write else None, cq, cache.k if cache.write else None)
             q = self.uq.forward(cq)
             qa = torch.empty((T, H * row), dtype=x.dtype, device=x.device)
-            ops.heads_matmul(q, Dn + Dr, self.uk, qa, row)
+            if self.uk_nt is not None and ops.heads_matmul_mfma_takes(q, Dn + Dr, self.uk_nt):
+                ops.heads_matmul_mfma(q, Dn + Dr, self.uk_nt, qa, row)
+            else:
+                ops.heads_matmul(q, Dn + Dr, self.uk, qa, row)
             if Dr:
                 ops.rotate_heads(q[:, Dn:], Dn + Dr, qa[:, Lk:], row, H, Dr, cos, sin, step.positions)
         latent = torch.empty((T, H * Lk), dtype=x.dtype, device=x.device)
@@ -154,5 +166,9 @@ class LatentAttention(Mixer):
             self._attend(qa, latent, step, cache, group)
         with profiling.label("o_proj", lambda: self.cost("o_proj", step, T)):
             out = torch.empty((T, H * Dv), dtype=x.dtype, device=x.device)
-            ops.heads_matmul(latent, Lk, self.uv, out, Dv, gate=low[:, Lq + row:] if self.output_gate else None)
+            gate = low[:, Lq + row:] if self.output_gate else None
+            if ops.heads_matmul_mfma_takes(latent, Lk, self.uv_nt):
+                ops.heads_matmul_mfma(latent, Lk, self.uv_nt, out, Dv, gate=gate)
+            else:
+                ops.heads_matmul(latent, Lk, self.uv, out, Dv, gate=gate)
             return self.o.forward(out)

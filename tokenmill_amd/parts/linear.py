@@ -60,6 +60,13 @@ class Linear(Part):
             self.packed = ops.pack_weight(w, rows() if callable(rows) else rows, parts)
             self._desc = None
 
+    def prepare(self, pack_weights: bool) -> None:
+        """A plain product by itself: the strip order the decode-step products read (one part; a stacked matrix whose
+        parts meet in an epilogue is packed by the part that owns it)."""
+        if pack_weights and self.packed is None and self.weight is not None and self.weight.dtype == torch.bfloat16 \
+                and self.weight.is_cuda and self.in_features % 8 == 0:
+            self.pack(lambda: ops.skinny_strip_rows(self.out_features, self.in_features))
+
     def describe(self):
         """The matrix, its packed copy and its bias as the kernel library takes them (kept until the tensors
         change); None while there is nothing on a GPU to describe."""

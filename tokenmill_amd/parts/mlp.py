@@ -99,6 +99,10 @@ class DenseFeedForward(FeedForward):
         if self.activation == "poly_norm":
             self.act = tensors[prefix + self.act_name].float().contiguous()
 
+    def prepare(self, pack_weights: bool) -> None:
+        self.up.prepare(pack_weights)
+        self.down.prepare(pack_weights)
+
     def cost(self, label: str, step: StepContext | None, rows: int) -> tuple[int, int]:
         return self.up.cost(rows) if label == "gate_up" else self.down.cost(rows)
 

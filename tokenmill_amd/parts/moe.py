@@ -72,5 +72,7 @@ class TableRoutedExperts(FeedForward):
         T = x.shape[0]
         out = torch.empty((T, self.hidden), dtype=x.dtype, device=x.device)
         with profiling.label("experts", lambda: self.cost("experts", step, T)):
-            routed = ops.moe_route(step.token_ids, self.table, self.experts)
+            mfma = x.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.intermediate % 8 == 0 and x.stride(0) % 8 == 0
+            rows = ops.moe_tile_rows(T * self.top, self.experts, x.dtype) if mfma else ops.MOE_TILE_ROWS
+            routed = ops.moe_route(step.token_ids, self.table, self.experts, rows)
             return ops.moe_experts(x, routed, self.gate_up, self.down, self.top, 1.0 / self.top, out)
