@@ -131,7 +131,7 @@ def test_poly_norm(dt, F):
 def test_products_head_by_head(dt, T, H, K, N):
     from tokenmill_amd.hip import ops
     torch.manual_seed(T + H)
-    pad_a, pad_c = (6, 4) if K % 8 else (8, 4)
+    pad_a, pad_c = (6, 4) if K % 8 else (8, 8)
     a = q(torch.randn(T, H * (K + pad_a)), dt)
     b = q(torch.randn(H, K, N) * 0.3, dt)
     gate = torch.randn(T, H + 3)
@@ -153,6 +153,19 @@ def test_products_head_by_head(dt, T, H, K, N):
         one = torch.zeros((1, H * (N + pad_c)), dtype=dt, device=DEV)
         ops.heads_matmul_mfma(ad[T // 2:T // 2 + 1], K + pad_a, wd, one, N + pad_c, gate=gate.to(DEV)[T // 2:T // 2 + 1, 2:])
         assert torch.equal(one.float().cpu().view(H, N + pad_c)[:, :N], got2[T // 2, :, :N])
+        # the channels behind a head's inputs go behind its outputs in the same launch, the first four rotated by position
+        from tokenmill_amd.parts import RotaryEmbedding
+        table = RotaryEmbedding(6, 1e4, 64, rotary_dim=4, interleaved=True)
+        table.build_tables(DEV)
+        pos = torch.arange(T) % 64
+        c3 = torch.full((T, H * (N + pad_c)), 7.0, dtype=dt, device=DEV)
+        ops.heads_matmul_mfma(ad, K + pad_a, wd, c3, N + pad_c, tail=6, cos=table.cos, sin=table.sin, positions=pos.to(torch.int32).to(DEV))
+        got3 = c3.float().cpu().view(T, H, N + pad_c)
+        plain = torch.einsum("thk,hkn->thn", a.view(T, H, K + pad_a)[..., :K], b)
+        close(got3[..., :N], q(plain, dt), dt, "per-head product beside a rotated tail")
+        turned = L.rotate_interleaved(a.view(T, H, K + pad_a)[..., K:K + 6], pos, 1e4, 4)
+        close(got3[..., N:N + 6], q(turned, dt), dt, "the rotated tail", bf16=2.0 ** -8)
+        assert bool((got3[..., N + 6:] == 7.0).all()), "wrote beyond the tail"
 
 
 def _experts_fixture(dt, width, ff, experts, top, vocab, seed):

@@ -220,7 +220,8 @@ int tm_moe_combine(const float* part, const int* pair_slot, void* y, int T, int 
 // [groups, N, K] with k contiguous. The *_takes functions say whether the operands come in whole 16-byte pieces.
 int tm_heads_matmul_mfma_takes(const void* A, int lda, int a_off, const void* W, int K);
 int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const void* W, void* C, int ldc, int c_off, const float* gate, int ldg,
-                         int T, int H, int K, int N, hipStream_t stream);
+                         int T, int H, int K, int N, int tail, int rot, const float* cos_t, const float* sin_t, const int* positions,
+                         hipStream_t stream);
 int tm_moe_mfma_takes(const void* x, int ldx, const void* Wgu, const void* Wd, const void* act, int K, int F);
 int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
                         const int* n_tiles, int max_tiles, int tile_rows, int K, int F, hipStream_t stream);

@@ -22,7 +22,9 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
                                                            const int* __restrict__ row_src, int src_div,
                                                            const bf16_t* __restrict__ W, void* __restrict__ Cv, int ldc, int c_off,
                                                            const float* __restrict__ gate, int ldg, const int* __restrict__ tiles,
-                                                           const int* __restrict__ n_tiles, int T, int K, int N) {
+                                                           const int* __restrict__ n_tiles, int T, int K, int N, int tail, int rot,
+                                                           const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                                           const int* __restrict__ positions) {
     constexpr int BM = RT * 16;
     constexpr bool GATED = MODE == GM_SILU_MUL;
     __shared__ __align__(16) bf16_t As[BM][GM_LD];
@@ -93,6 +95,25 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
         }
         __syncthreads();
     }
+    // heads: the `tail` channels that follow a head's K input channels go behind its N output channels, their first `rot`
+    // rotated in pairs (2i, 2i + 1) by the row's position (the rotated part of a query head beside its part on the latent)
+    if (MODE == GM_STORE && tail > 0 && blockIdx.y == 0) {
+        const int half = rot / 2, rest = tail - rot;
+        for (int idx = threadIdx.x; idx < rows * half; idx += 256) {
+            const int row = row0 + idx / half, c = idx % half;
+            const bf16_t* sp = A + (size_t)row * lda + (size_t)group * a_off + K + 2 * c;
+            bf16_t* dp = (bf16_t*)Cv + (size_t)row * ldc + (size_t)group * c_off + N + 2 * c;
+            const size_t at = (size_t)positions[row] * half + c;
+            float a, b;
+            rotate_pair(bf16_to_f32(sp[0]), bf16_to_f32(sp[1]), cos_t[at], sin_t[at], a, b);
+            dp[0] = f32_to_bf16(a);
+            dp[1] = f32_to_bf16(b);
+        }
+        for (int idx = threadIdx.x; idx < rows * rest; idx += 256) {
+            const int row = row0 + idx / rest, c = rot + idx % rest;
+            ((bf16_t*)Cv)[(size_t)row * ldc + (size_t)group * c_off + N + c] = A[(size_t)row * lda + (size_t)group * a_off + K + c];
+        }
+    }
     const int n = n0 + 16 * wave + r;
     if (n >= N) return;
 #pragma unroll
@@ -123,16 +144,20 @@ extern "C" int tm_heads_matmul_mfma_takes(const void* A, int lda, int a_off, con
 }
 
 // C[t, h * c_off + n] = sum_k A[t, h * a_off + k] * W[h][n][k] (W [H, N, K]), times sigmoid(gate[t * ldg + h]) if gate.
+// tail > 0: also C[t, h * c_off + N + c] = A[t, h * a_off + K + c] for c < tail, the first `rot` of them rotated in pairs
+// (2i, 2i + 1) by positions[t] (cos_t, sin_t [positions, rot / 2]).
 extern "C" int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const void* W, void* C, int ldc, int c_off, const float* gate,
-                                    int ldg, int T, int H, int K, int N, hipStream_t stream) {
-    if (!A || !W || !C || T < 0 || H <= 0 || H > 65535 || K <= 0 || N <= 0 || a_off < K || c_off < N ||
-        !tm_heads_matmul_mfma_takes(A, lda, a_off, W, K) || (gate && ldg < H))
+                                    int ldg, int T, int H, int K, int N, int tail, int rot, const float* cos_t, const float* sin_t,
+                                    const int* positions, hipStream_t stream) {
+    if (!A || !W || !C || T < 0 || H <= 0 || H > 65535 || K <= 0 || N <= 0 || tail < 0 || rot < 0 || rot > tail || rot % 2 ||
+        a_off < K + tail || c_off < N + tail || !tm_heads_matmul_mfma_takes(A, lda, a_off, W, K) || (gate && ldg < H) ||
+        (rot && (!cos_t || !sin_t || !positions)))
         return TM_ERR_ARG;
     if (T == 0) return TM_OK;
     dim3 grid((T + 63) / 64, (N + GM_BN - 1) / GM_BN, H);
     if (grid.y > 65535) return TM_ERR_ARG;
     grouped_mfma_kernel<4, GM_STORE><<<grid, 256, 0, stream>>>((const bf16_t*)A, lda, a_off, nullptr, 1, (const bf16_t*)W, C, ldc, c_off,
-                                                               gate, ldg, nullptr, nullptr, T, K, N);
+                                                               gate, ldg, nullptr, nullptr, T, K, N, tail, rot, cos_t, sin_t, positions);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
@@ -154,7 +179,7 @@ extern "C" int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair,
     if (grid.y > 65535) return TM_ERR_ARG;
 #define GM_GO(RT_)                                                                                                             \
     grouped_mfma_kernel<RT_, GM_SILU_MUL><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
-                                                                    0, nullptr, 0, tiles, n_tiles, 0, K, F)
+                                                                    0, nullptr, 0, tiles, n_tiles, 0, K, F, 0, 0, nullptr, nullptr, nullptr)
     if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
 #undef GM_GO
     TM_CHECK_LAUNCH();
@@ -171,7 +196,7 @@ extern "C" int tm_moe_down_mfma(const void* act, const void* W, float* part, con
     if (grid.y > 65535) return TM_ERR_ARG;
 #define GM_GO(RT_)                                                                                                              \
     grouped_mfma_kernel<RT_, GM_STORE_F32><<<grid, 256, 0, stream>>>((const bf16_t*)act, F, 0, nullptr, 1, (const bf16_t*)W, part, N, 0, \
-                                                                     nullptr, 0, tiles, n_tiles, 0, F, N)
+                                                                     nullptr, 0, tiles, n_tiles, 0, F, N, 0, 0, nullptr, nullptr, nullptr)
     if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
 #undef GM_GO
     TM_CHECK_LAUNCH();

@@ -1444,18 +1444,25 @@ def heads_matmul_mfma_takes(a: torch.Tensor, a_head: int, w: torch.Tensor) -> bo
 
 
 def heads_matmul_mfma(a: torch.Tensor, a_head: int, w: torch.Tensor, c: torch.Tensor, c_head: int,
-                      gate: torch.Tensor | None = None) -> torch.Tensor:
+                      gate: torch.Tensor | None = None, tail: int = 0, cos: torch.Tensor | None = None,
+                      sin: torch.Tensor | None = None, positions: torch.Tensor | None = None) -> torch.Tensor:
     """``heads_matmul`` on the matrix unit, with the matrices given as w [H, N, K] (k contiguous): c[t, h * c_head + n] =
-    sum_k a[t, h * a_head + k] * w[h, n, k], times sigmoid(gate[t, h]) if ``gate`` (float32 [T, >= H])."""
+    sum_k a[t, h * a_head + k] * w[h, n, k], times sigmoid(gate[t, h]) if ``gate`` (float32 [T, >= H]). ``tail`` > 0: the
+    ``tail`` channels behind a head's K input channels are copied behind its N output channels, the first 2 * cos.shape[1]
+    of them rotated in pairs (2i, 2i + 1) by the row's position (``rotate_heads`` in the same launch)."""
     _gpu(a, w, c, gate)
     T = a.shape[0]
     H, N, K = w.shape
     _need(a.dim() == 2 and c.dim() == 2 and a.stride(1) == 1 and c.stride(1) == 1 and c.shape[0] == T and w.is_contiguous(),
           "heads_matmul: a, c [T, .] with unit inner stride, w contiguous [H, N, K]")
     _need(a.dtype == w.dtype == c.dtype == torch.bfloat16, "heads_matmul (matrix unit): bfloat16")
-    _need(a_head >= K and c_head >= N and a.shape[1] >= (H - 1) * a_head + K and c.shape[1] >= (H - 1) * c_head + N,
-          "heads_matmul: the heads do not fit the rows")
+    _need(tail >= 0 and a_head >= K + tail and c_head >= N + tail and a.shape[1] >= (H - 1) * a_head + K + tail
+          and c.shape[1] >= (H - 1) * c_head + N + tail, "heads_matmul: the heads do not fit the rows")
     _need(heads_matmul_mfma_takes(a, a_head, w), "heads_matmul (matrix unit): operands not in whole 16-byte pieces")
+    rot = 2 * cos.shape[1] if (cos is not None and tail) else 0
+    _need(rot <= tail, "heads_matmul: more rotated channels than the tail has")
+    _angles(cos, sin, rot, positions, T, "heads_matmul")
+    _gpu(cos, sin, positions)
     gate_stride = 0
     if gate is not None:
         _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= H and gate.stride(1) == 1,
@@ -1464,7 +1471,9 @@ def heads_matmul_mfma(a: torch.Tensor, a_head: int, w: torch.Tensor, c: torch.Te
     lda = a.stride(0) if T > 1 else max(a.stride(0), a.shape[1])
     ldc = c.stride(0) if T > 1 else max(c.stride(0), c.shape[1])
     _check(library().tm_heads_matmul_mfma(_p(a), c_int(lda), c_int(a_head), _p(w), _p(c), c_int(ldc), c_int(c_head), _p(gate),
-                                          c_int(gate_stride), c_int(T), c_int(H), c_int(K), c_int(N), _stream()), "heads_matmul_mfma")
+                                          c_int(gate_stride), c_int(T), c_int(H), c_int(K), c_int(N), c_int(tail), c_int(rot),
+                                          _p(cos if rot else None), _p(sin if rot else None), _p(positions if rot else None), _stream()),
+           "heads_matmul_mfma")
     return c
 
 

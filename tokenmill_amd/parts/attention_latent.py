@@ -156,11 +156,12 @@ class LatentAttention(Mixer):
             q = self.uq.forward(cq)
             qa = torch.empty((T, H * row), dtype=x.dtype, device=x.device)
             if self.uk_nt is not None and ops.heads_matmul_mfma_takes(q, Dn + Dr, self.uk_nt):
-                ops.heads_matmul_mfma(q, Dn + Dr, self.uk_nt, qa, row)
+                # the heads' rotated channels go beside their part on the latent in the same launch
+                ops.heads_matmul_mfma(q, Dn + Dr, self.uk_nt, qa, row, tail=Dr, cos=cos, sin=sin, positions=step.positions)
             else:
                 ops.heads_matmul(q, Dn + Dr, self.uk, qa, row)
-            if Dr:
-                ops.rotate_heads(q[:, Dn:], Dn + Dr, qa[:, Lk:], row, H, Dr, cos, sin, step.positions)
+                if Dr:
+                    ops.rotate_heads(q[:, Dn:], Dn + Dr, qa[:, Lk:], row, H, Dr, cos, sin, step.positions)
         latent = torch.empty((T, H * Lk), dtype=x.dtype, device=x.device)
         with profiling.label("attention", lambda: self.cost("attention", step, T)):
             self._attend(qa, latent, step, cache, group)
