@@ -88,7 +88,7 @@ def test_short_convolution_whole_cut_and_beside_another_request(dt, taps, width)
     state = state.contiguous() if taps > 1 else None
     wd = w.to(dt).to(DEV)
 
-    def run(pieces):          # pieces: [(rows of a, rows of b)] per step; a in slot 2, b in slot 0
+    def run(pieces, walk=True):   # pieces: [(rows of a, rows of b)] per step; a in slot 2, b in slot 0; walk: one launch where rows are few
         if state is not None:
             state[2].zero_(), state[0].zero_()
         outs_a, outs_b, pa, pb = [], [], 0, 0
@@ -99,7 +99,8 @@ def test_short_convolution_whole_cut_and_beside_another_request(dt, taps, width)
             for n, _ in seqs:
                 cu.append(cu[-1] + n)
             seq_of = [i for i, (n, _) in enumerate(seqs) for _ in range(n)]
-            out = ops.short_conv(h, wd, state, ints(cu), ints([s for _, s in seqs]), ints(seq_of), len(seqs), torch.empty_like(h))
+            out = ops.short_conv(h, wd, state, ints(cu), ints([s for _, s in seqs]), ints(seq_of), len(seqs), torch.empty_like(h),
+                                 most_rows=max(na, nb) if walk else 0)
             outs_a.append(out[:na].float().cpu())
             outs_b.append(out[na:].float().cpu())
             pa, pb = pa + na, pb + nb
@@ -110,8 +111,9 @@ def test_short_convolution_whole_cut_and_beside_another_request(dt, taps, width)
         close(a, q(want_a, dt), dt, f"request a in {len(pieces)} steps", bf16=2.0 ** -8)
         close(b, q(want_b, dt), dt, f"request b in {len(pieces)} steps", bf16=2.0 ** -8)
     first = run([(23, 9)])
-    again = run([(5, 4), (18, 5)])
-    assert torch.equal(first[0], again[0]) and torch.equal(first[1], again[1]), "a cut changes bits"
+    for pieces, walk in (([(5, 4), (18, 5)], True), ([(1, 1)] * 9 + [(1, 0)] * 14, True), ([(1, 1)] * 9 + [(1, 0)] * 14, False)):
+        again = run(pieces, walk)
+        assert torch.equal(first[0], again[0]) and torch.equal(first[1], again[1]), "a cut changes bits"
 
 
 @pytest.mark.parametrize("dt", DTS)
@@ -283,13 +285,13 @@ def test_latent_attention_whole_in_portions_and_token_by_token(dt, H, Dn, Dr, Dv
 
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("window,page", [(24, 8), (17, 16), (33, 4)])
-def test_rows_just_inside_and_just_outside_the_window_show(dt, window, page):
+@pytest.mark.parametrize("window,page,H", [(24, 8, 5), (17, 16, 20), (33, 4, 70), (64, 32, 16)])
+def test_rows_just_inside_and_just_outside_the_window_show(dt, window, page, H):
     """Cached rows whose latent is one channel set to one (row j sets channel j % Lk) and whose scores are all equal: a
     token's result is then, channel by channel, how many visible rows set that channel, over the number of visible rows.
     One row too many or too few, at the window's far edge or at the token itself, changes both."""
     from tokenmill_amd.hip import ops
-    H, Lk, Dr = 5, 40, 8
+    Lk, Dr = 40, 8
     Dk = Lk + Dr
     n = 90
     pool = torch.zeros((n // page + 2, page, 1, Dk), dtype=dt, device=DEV)

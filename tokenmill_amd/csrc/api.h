@@ -177,6 +177,8 @@ int tm_layer_norm(float* resid, const void* y, const void* gate, float mult, con
 // taps - 1 rows the request has seen. h, out, w [width, taps] and state of type `dtype`; taps up to 16.
 int tm_short_conv(const void* h, void* out, const void* w, const void* state, const int* cu_q_lens, const int* state_slots,
                   const int* seq_of_token, int T, int width, int taps, int dtype, hipStream_t stream);
+int tm_short_conv_walk(const void* h, void* out, const void* w, void* state, const int* cu_q_lens, const int* state_slots, int S,
+                       int width, int taps, int dtype, hipStream_t stream);
 int tm_short_conv_state(const void* h, void* state, const int* cu_q_lens, const int* state_slots, int S, int width, int taps,
                         int dtype, hipStream_t stream);
 // out = a N(z) + b N(z^2) + c N(z^3) + e with coef = (a, b, c, e) on the device, N(v) = v / sqrt(mean(v^2) + eps) per row.

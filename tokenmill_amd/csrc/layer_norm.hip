@@ -8,6 +8,7 @@
 //   tm_short_conv      out[t] = h[t] + sum_j w[:, j] * h[t - taps + 1 + j], the rows before a request's first row of the
 //                      step taken from its state [taps - 1, width] (zeros at a sequence's start);
 //   tm_short_conv_state  then the state becomes the last taps - 1 rows the request has seen.
+//   tm_short_conv_walk   both in one launch, for steps whose requests bring few rows each; the same bits.
 //   tm_poly_norm       out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over a row, powers by element.
 #include "common.h"
 #include "api.h"
@@ -70,7 +71,19 @@ extern "C" int tm_layer_norm(float* resid, const void* y, const void* gate, floa
 #define SC_THREADS 256
 #define SC_MAX_TAPS 16
 
-template <typename T>
+// sum_j w[j] * x[j], j ascending, every product and sum rounded on its own: the two kernels below give the same bits
+// (MAXT: the most taps the instantiation takes; the sum is the same sequence of operations at every MAXT)
+template <int MAXT>
+__device__ __forceinline__ float tap_sum(const float (&wv)[MAXT], const float (&xv)[MAXT], int taps) {
+#pragma clang fp contract(off)
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < MAXT; ++j)
+        if (j < taps) acc += wv[j] * xv[j];
+    return acc;
+}
+
+template <typename T, int MAXT>
 __global__ __launch_bounds__(SC_THREADS) void short_conv_kernel(const T* __restrict__ h, T* __restrict__ out,
                                                                 const T* __restrict__ w, const T* __restrict__ state,
                                                                 const int* __restrict__ cu, const int* __restrict__ slots,
@@ -81,14 +94,52 @@ __global__ __launch_bounds__(SC_THREADS) void short_conv_kernel(const T* __restr
     const int i = t - first;                                 // the token's place among its request's rows of this step
     const T* st = state + (size_t)slots[s] * (taps - 1) * width;
     for (int c = blockIdx.y * SC_THREADS + threadIdx.x; c < width; c += gridDim.y * SC_THREADS) {
-        float acc = 0.f;
-        for (int j = 0; j < taps; ++j) {
-            const int at = i - (taps - 1) + j;               // < 0: before this step's rows, in the state
-            const float v = at >= 0 ? Elem<T>::load(h + (size_t)(first + at) * width + c)
-                                    : Elem<T>::load(st + (size_t)(taps - 1 + at) * width + c);
-            acc += Elem<T>::load(w + (size_t)c * taps + j) * v;
+        float wv[MAXT], xv[MAXT];
+#pragma unroll
+        for (int j = 0; j < MAXT; ++j) {
+            wv[j] = xv[j] = 0.f;
+            if (j < taps) {
+                const int at = i - (taps - 1) + j;           // < 0: before this step's rows, in the state
+                xv[j] = at >= 0 ? Elem<T>::load(h + (size_t)(first + at) * width + c)
+                                : Elem<T>::load(st + (size_t)(taps - 1 + at) * width + c);
+                wv[j] = Elem<T>::load(w + (size_t)c * taps + j);
+            }
         }
-        Elem<T>::store(out + (size_t)t * width + c, Elem<T>::load(h + (size_t)t * width + c) + acc);
+        Elem<T>::store(out + (size_t)t * width + c, Elem<T>::load(h + (size_t)t * width + c) + tap_sum<MAXT>(wv, xv, taps));
+    }
+}
+
+// The same for steps whose requests bring few rows each (single tokens): a thread takes a channel of a request, walks the
+// request's rows with the window of the last taps rows in registers, and leaves the new state behind: one launch.
+template <typename T, int MAXT>
+__global__ __launch_bounds__(SC_THREADS) void short_conv_walk_kernel(const T* __restrict__ h, T* __restrict__ out,
+                                                                     const T* __restrict__ w, T* __restrict__ state,
+                                                                     const int* __restrict__ cu, const int* __restrict__ slots,
+                                                                     int width, int taps) {
+    const int s = blockIdx.x;
+    const int first = cu[s], n = cu[s + 1] - first;
+    if (n <= 0) return;
+    T* st = state + (size_t)slots[s] * (taps - 1) * width;
+    for (int c = blockIdx.y * SC_THREADS + threadIdx.x; c < width; c += gridDim.y * SC_THREADS) {
+        float wv[MAXT], xv[MAXT];
+#pragma unroll
+        for (int j = 0; j < MAXT; ++j) {
+            wv[j] = j < taps ? Elem<T>::load(w + (size_t)c * taps + j) : 0.f;
+            xv[j] = j < taps - 1 ? Elem<T>::load(st + (size_t)j * width + c) : 0.f;
+        }
+        for (int i = 0; i < n; ++i) {
+            const float cur = Elem<T>::load(h + (size_t)(first + i) * width + c);
+#pragma unroll
+            for (int j = 0; j < MAXT; ++j)
+                if (j == taps - 1) xv[j] = cur;
+            Elem<T>::store(out + (size_t)(first + i) * width + c, cur + tap_sum<MAXT>(wv, xv, taps));
+#pragma unroll
+            for (int j = 0; j + 1 < MAXT; ++j)
+                if (j < taps - 1) xv[j] = xv[j + 1];
+        }
+#pragma unroll
+        for (int j = 0; j < MAXT; ++j)
+            if (j < taps - 1) Elem<T>::store(st + (size_t)j * width + c, xv[j]);
     }
 }
 
@@ -118,13 +169,35 @@ extern "C" int tm_short_conv(const void* h, void* out, const void* w, const void
     if (dtype != TM_F32 && dtype != TM_BF16) return TM_ERR_ARG;
     if (T == 0) return TM_OK;
     dim3 grid(T, (width + SC_THREADS - 1) / SC_THREADS > 8 ? 8 : (width + SC_THREADS - 1) / SC_THREADS);
-    if (dtype == TM_F32)
-        short_conv_kernel<float><<<grid, SC_THREADS, 0, stream>>>((const float*)h, (float*)out, (const float*)w, (const float*)state,
-                                                                  cu_q_lens, state_slots, seq_of_token, width, taps);
-    else
-        short_conv_kernel<bf16_t><<<grid, SC_THREADS, 0, stream>>>((const bf16_t*)h, (bf16_t*)out, (const bf16_t*)w,
-                                                                   (const bf16_t*)state, cu_q_lens, state_slots, seq_of_token,
-                                                                   width, taps);
+#define SC_GO(T_, MAXT_)                                                                                                  \
+    short_conv_kernel<T_, MAXT_><<<grid, SC_THREADS, 0, stream>>>((const T_*)h, (T_*)out, (const T_*)w, (const T_*)state, cu_q_lens, \
+                                                                  state_slots, seq_of_token, width, taps)
+    if (dtype == TM_F32) {
+        if (taps <= 4) SC_GO(float, 4); else if (taps <= 8) SC_GO(float, 8); else SC_GO(float, SC_MAX_TAPS);
+    } else {
+        if (taps <= 4) SC_GO(bf16_t, 4); else if (taps <= 8) SC_GO(bf16_t, 8); else SC_GO(bf16_t, SC_MAX_TAPS);
+    }
+#undef SC_GO
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// tm_short_conv and tm_short_conv_state in one launch, for steps whose requests bring few rows each: the same bits.
+extern "C" int tm_short_conv_walk(const void* h, void* out, const void* w, void* state, const int* cu_q_lens, const int* state_slots,
+                                  int S, int width, int taps, int dtype, hipStream_t stream) {
+    if (!h || !out || !w || S < 0 || width <= 0 || taps < 2 || taps > SC_MAX_TAPS || !state) return TM_ERR_ARG;
+    if (dtype != TM_F32 && dtype != TM_BF16) return TM_ERR_ARG;
+    if (S == 0) return TM_OK;
+    dim3 grid(S, (width + SC_THREADS - 1) / SC_THREADS > 8 ? 8 : (width + SC_THREADS - 1) / SC_THREADS);
+#define SC_GO(T_, MAXT_)                                                                                                       \
+    short_conv_walk_kernel<T_, MAXT_><<<grid, SC_THREADS, 0, stream>>>((const T_*)h, (T_*)out, (const T_*)w, (T_*)state, cu_q_lens,     \
+                                                                       state_slots, width, taps)
+    if (dtype == TM_F32) {
+        if (taps <= 4) SC_GO(float, 4); else if (taps <= 8) SC_GO(float, 8); else SC_GO(float, SC_MAX_TAPS);
+    } else {
+        if (taps <= 4) SC_GO(bf16_t, 4); else if (taps <= 8) SC_GO(bf16_t, 8); else SC_GO(bf16_t, SC_MAX_TAPS);
+    }
+#undef SC_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

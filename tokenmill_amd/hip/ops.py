@@ -1321,11 +1321,16 @@ def layer_norm(resid: torch.Tensor, y: torch.Tensor | None, gate: torch.Tensor |
     return out
 
 
+SHORT_CONV_WALK_ROWS = 8        # up to this many rows a request, a step's convolution and its new state are one launch
+
+
 def short_conv(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor | None, cu_q_lens: torch.Tensor, state_slots: torch.Tensor,
-               seq_of_token: torch.Tensor, num_seqs: int, out: torch.Tensor) -> torch.Tensor:
+               seq_of_token: torch.Tensor, num_seqs: int, out: torch.Tensor, most_rows: int = 0) -> torch.Tensor:
     """out[t] = h[t] + sum_j w[:, j] * h[t - taps + 1 + j] within each request (rows cu_q_lens[s] .. cu_q_lens[s + 1] - 1 of h),
     the rows before the step's first taken from state[state_slots[s]] ([taps - 1, width]); afterwards that state holds the
-    last taps - 1 rows the request has seen. h, w [width, taps], state [slots, taps - 1, width] and out share one type."""
+    last taps - 1 rows the request has seen. h, w [width, taps], state [slots, taps - 1, width] and out share one type.
+    ``most_rows``: the most rows any request brings, if known: few rows a request (single tokens) take one launch in which a
+    thread walks a request's rows, otherwise the convolution and the state's update are two; both give the same bits."""
     _gpu(h, w, state, cu_q_lens, state_slots, seq_of_token, out)
     T, width = h.shape
     taps = w.shape[1]
@@ -1340,6 +1345,10 @@ def short_conv(h: torch.Tensor, w: torch.Tensor, state: torch.Tensor | None, cu_
     _ints(state_slots, num_seqs, "state_slots")
     _ints(seq_of_token, T, "seq_of_token")
     lib = library()
+    if taps > 1 and 0 < most_rows <= SHORT_CONV_WALK_ROWS:
+        _check(lib.tm_short_conv_walk(_p(h), _p(out), _p(w), _p(state), _p(cu_q_lens), _p(state_slots), c_int(num_seqs), c_int(width),
+                                      c_int(taps), c_int(code(h.dtype)), _stream()), "short_conv_walk")
+        return out
     _check(lib.tm_short_conv(_p(h), _p(out), _p(w), _p(state), _p(cu_q_lens), _p(state_slots), _p(seq_of_token), c_int(T),
                              c_int(width), c_int(taps), c_int(code(h.dtype)), _stream()), "short_conv")
     if taps > 1:

@@ -42,4 +42,5 @@ class ShortConvolution(Part):
         """h [T, width] -> h + conv(h), request by request; ``state`` [slots, taps - 1, width] is read and advanced."""
         out = torch.empty_like(h)
         with profiling.label("conv", lambda: self.cost("conv", step, h.shape[0])):
-            return ops.short_conv(h, self.weight, state, step.cu_q_lens, step.state_slots, step.seq_of_token, step.num_seqs, out)
+            return ops.short_conv(h, self.weight, state, step.cu_q_lens, step.state_slots, step.seq_of_token, step.num_seqs, out,
+                                  most_rows=step.max_q_len)
