@@ -59,16 +59,18 @@ def build_lusolix(cfg: LusolixConfig, max_positions: int | None = None) -> Decod
                                places=LearnedPositions(cfg.max_position_embeddings, hidden, name="pos"))
     tables: dict = {}
     layers = []
-    for layer in cfg.layers:
+    unused: list[str] = []              # what a checkpoint may hold for a sublayer that a layer does not have
+    for i, layer in enumerate(cfg.layers):
         conv = ShortConvolution(hidden, cfg.conv_taps, name="canon1") if cfg.conv_taps else None
         mixer = _mixer(cfg, layer, n_pos, tables)
         if layer.mlp is None:
+            unused += [f"l{i}.norm2", f"l{i}.norm2.b", f"l{i}.rg2", f"l{i}.rg2.b"]
             layers.append(GatedResidualBlock(norm(), mixer, gate_mixed=gate("rg1"), conv=conv, mult=cfg.residual_mult))
         else:
             layers.append(GatedResidualBlock(norm(), mixer, norm(), _feed_forward(cfg, layer.mlp), gate("rg1"), gate("rg2"), conv,
                                              cfg.residual_mult))
     head = OutputHead(hidden, cfg.vocab_size, tied_to=embedding, name="head", suffixes=SUFFIXES)
-    return DecoderModel(cfg, embedding, layers, norm(), head, names=("", "l{i}.", "final.norm", ""))
+    return DecoderModel(cfg, embedding, layers, norm(), head, names=("", "l{i}.", "final.norm", ""), ignorable=tuple(unused))
 
 
 register_architecture(LusolixConfig.architecture, LusolixConfig.from_dict, build_lusolix, replace=True)
