@@ -19,13 +19,15 @@
 #include "attention_prefill_common.h"
 
 #define LM_KEYS 32
-#define LM_PAD 8
-#define LM_VT_STRIDE (LM_KEYS + LM_PAD)
+#define LM_PAD 16               // staged rows lie 32 bytes more than a multiple of 64 apart: their 16-byte operand loads meet no bank twice
+#define LM_VT_STRIDE (LM_KEYS + 8)
 #define LM_MAX_CHUNKS 64        // a single token's visible rows are dealt to about this many blocks at most
 
-// WAVES: wavefronts (= tiles) of a block. NDT: tiles of 16 latent channels a wavefront may hold (Lk <= 16 NDT).
-// NDC: chunks of 32 channels of a cached row it may hold (Dk <= 32 NDC).
-template <int WAVES, int NDT, int NDC>
+// WAVES: wavefronts of a block; SPLIT of them share a tile of pairs, each with its own part of the latent's channels (a wide
+// latent's results of one tile do not fit a wavefront's registers beside a second wavefront on the SIMD; halved they do, and
+// two wavefronts a SIMD hide each other's waits. Both compute the tile's scores). NDT: tiles of 16 latent channels a tile of
+// pairs may have (Lk <= 16 NDT). NDC: chunks of 32 channels of a cached row (Dk <= 32 NDC).
+template <int WAVES, int NDT, int NDC, int SPLIT>
 __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
     const bf16_t* __restrict__ qa, int q_stride, bf16_t* __restrict__ out, int out_stride, const bf16_t* __restrict__ pool,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ tiles, int head_groups,
@@ -39,17 +41,19 @@ __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TM_WAVE);
     const int lane = threadIdx.x % TM_WAVE, r = lane % 16, g = lane / 16;
     const bool single = tiles == nullptr;
+    constexpr int TILES = WAVES / SPLIT, NDTP = NDT / SPLIT;              // tiles of pairs a block; channel tiles a wavefront
+    const int d0 = (wave % SPLIT) * NDTP;                                 // this wavefront's first channel tile
 
     int s, row0, valid, pos0, tile_head;
     if (!single) {
         const int* tl = tiles + (size_t)(blockIdx.x / head_groups) * 4;
         s = tl[0], row0 = tl[1], valid = tl[2], pos0 = tl[3];
-        tile_head = (blockIdx.x % head_groups) * WAVES + wave;           // this wavefront's head
+        tile_head = (blockIdx.x % head_groups) * TILES + wave / SPLIT;   // this wavefront's head
     } else {
         row0 = first_single + blockIdx.x / head_groups;
         s = seq_of_token[row0];
         pos0 = positions[row0];
-        tile_head = ((blockIdx.x % head_groups) * WAVES + wave) * 16;    // its first head
+        tile_head = ((blockIdx.x % head_groups) * TILES + wave / SPLIT) * 16;    // its first head
         valid = 1;
     }
     const bool tile_ok = tile_head < H;                                   // wave-uniform
@@ -80,9 +84,9 @@ __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
             qf[c].u = u32x4_t{0, 0, 0, 0};
     }
     float m = -INFINITY, l = 0.f;
-    f32x4_t o[NDT];
+    f32x4_t o[NDTP];
 #pragma unroll
-    for (int d = 0; d < NDT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int d = 0; d < NDTP; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     const int pieces = DKP / 8;                                           // 16-byte pieces of a staged row
     // Consecutive lanes take consecutive rows (the transposed copy is then written without bank conflicts), so a thread keeps
@@ -170,10 +174,10 @@ __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
         pt.u = u32x4_t{pk_bf16(pr[0][0], pr[0][1]), pk_bf16(pr[0][2], pr[0][3]), pk_bf16(pr[1][0], pr[1][1]),
                        pk_bf16(pr[1][2], pr[1][3])};
 #pragma unroll
-        for (int d = 0; d < NDT; ++d) {
-            if (16 * d >= Lk) continue;
+        for (int d = 0; d < NDTP; ++d) {
+            if (16 * (d0 + d) >= Lk) continue;                            // wave-uniform
             o[d] *= alpha;
-            const bf16_t* vrow = Vt + (16 * d + r) * LM_VT_STRIDE + 4 * g;
+            const bf16_t* vrow = Vt + (16 * (d0 + d) + r) * LM_VT_STRIDE + 4 * g;
             const u32x2_t v0 = *(const u32x2_t*)vrow, v1 = *(const u32x2_t*)(vrow + 16);
             PFrag vf;
             vf.u = u32x4_t{v0[0], v0[1], v1[0], v1[1]};
@@ -187,14 +191,14 @@ __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
     if (!pair_ok) return;
     if (part_o) {                                                         // a chunk's share: as it is, with its maximum and sum
         const size_t at = ((size_t)(row0 - first_single) * H + head) * n_chunks + blockIdx.y;
-        if (g == 0) {
+        if (g == 0 && wave % SPLIT == 0) {
             part_ml[2 * at] = m;
             part_ml[2 * at + 1] = total;
         }
         float* dst = part_o + at * Lk;
 #pragma unroll
-        for (int d = 0; d < NDT; ++d) {
-            const int ch = 16 * d + 4 * g;
+        for (int d = 0; d < NDTP; ++d) {
+            const int ch = 16 * (d0 + d) + 4 * g;
             if (ch < Lk) *(f32x4_t*)(dst + ch) = o[d];
         }
         return;
@@ -202,8 +206,8 @@ __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
     const float inv = 1.0f / total;
     bf16_t* dst = out + (size_t)token * out_stride + (size_t)head * Lk;
 #pragma unroll
-    for (int d = 0; d < NDT; ++d) {
-        const int ch = 16 * d + 4 * g;
+    for (int d = 0; d < NDTP; ++d) {
+        const int ch = 16 * (d0 + d) + 4 * g;
         if (ch < Lk) *(u32x2_t*)(dst + ch) = u32x2_t{pk_bf16(o[d][0] * inv, o[d][1] * inv), pk_bf16(o[d][2] * inv, o[d][3] * inv)};
     }
 }
@@ -271,9 +275,9 @@ struct LmArgs {
     float* part_ml; int n_chunks; int chunk_runs; int H, Lk, Dk, page; float scale_log2; int window;
 };
 
-template <int WAVES, int NDT, int NDC>
+template <int WAVES, int NDT, int NDC, int SPLIT>
 static int lm_launch(dim3 grid, size_t lds, hipStream_t stream, const LmArgs& a) {
-    auto kernel = attn_latent_mfma_kernel<WAVES, NDT, NDC>;
+    auto kernel = attn_latent_mfma_kernel<WAVES, NDT, NDC, SPLIT>;
     static size_t allowed = 64 * 1024;                                   // per instantiation: the most LDS asked for so far
     if (lds > allowed) {
         if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
@@ -286,16 +290,16 @@ static int lm_launch(dim3 grid, size_t lds, hipStream_t stream, const LmArgs& a)
     return TM_OK;
 }
 
-template <int WAVES>
+// a latent of more than 256 channels: eight wavefronts a block, two a tile of pairs; four tiles a block either way
 static int lm_pick(dim3 grid, size_t lds, hipStream_t stream, const LmArgs& a) {
     const int ndt = (a.Lk + 15) / 16, ndc = (a.Dk + 31) / 32;
-#define LM_ROW(NDT_)                                                              \
-    if (ndc <= 4) return lm_launch<WAVES, NDT_, 4>(grid, lds, stream, a);         \
-    if (ndc <= 10) return lm_launch<WAVES, NDT_, 10>(grid, lds, stream, a);       \
-    return lm_launch<WAVES, NDT_, 22>(grid, lds, stream, a);
-    if (ndt <= 8) { LM_ROW(8) }
-    if (ndt <= 16) { LM_ROW(16) }
-    LM_ROW(32)
+#define LM_ROW(WAVES_, NDT_, SPLIT_)                                                         \
+    if (ndc <= 4) return lm_launch<WAVES_, NDT_, 4, SPLIT_>(grid, lds, stream, a);           \
+    if (ndc <= 10) return lm_launch<WAVES_, NDT_, 10, SPLIT_>(grid, lds, stream, a);         \
+    return lm_launch<WAVES_, NDT_, 22, SPLIT_>(grid, lds, stream, a);
+    if (ndt <= 8) { LM_ROW(4, 8, 1) }
+    if (ndt <= 16) { LM_ROW(4, 16, 1) }
+    LM_ROW(8, 32, 2)
 #undef LM_ROW
 }
 
@@ -325,14 +329,14 @@ extern "C" int tm_attn_latent_mfma(const void* qa, int q_stride, void* out, int 
         a.head_groups = (H + 3) / 4;
         const long long blocks = (long long)n_tiles * a.head_groups;
         if (blocks > 0x7fffffffLL) return TM_ERR_ARG;
-        rc = lm_pick<4>(dim3((unsigned)blocks), lds, stream, a);
+        rc = lm_pick(dim3((unsigned)blocks), lds, stream, a);
     } else {
         a.head_groups = (H + 63) / 64;                                    // four wavefronts stage a run together; each takes 16 heads
         a.part_o = part_o;
         a.part_ml = part_ml;
         const long long blocks = (long long)n_single * a.head_groups;
         if (blocks > 0x7fffffffLL) return TM_ERR_ARG;
-        rc = lm_pick<4>(dim3((unsigned)blocks, n_chunks), lds, stream, a);
+        rc = lm_pick(dim3((unsigned)blocks, n_chunks), lds, stream, a);
         if (rc == TM_OK) {
             TM_CHECK_LAUNCH();
             attn_latent_merge_kernel<<<n_single * H, 128, (size_t)n_chunks * sizeof(float), stream>>>(part_o, part_ml, (bf16_t*)out, out_stride, first_single, H, Lk,
