@@ -290,7 +290,7 @@ static int lm_launch(dim3 grid, size_t lds, hipStream_t stream, const LmArgs& a)
     return TM_OK;
 }
 
-// a latent of more than 256 channels: eight wavefronts a block, two a tile of pairs; four tiles a block either way
+// a latent of more than 128 channels: eight wavefronts a block, two a tile of pairs; four tiles a block either way
 static int lm_pick(dim3 grid, size_t lds, hipStream_t stream, const LmArgs& a) {
     const int ndt = (a.Lk + 15) / 16, ndc = (a.Dk + 31) / 32;
 #define LM_ROW(WAVES_, NDT_, SPLIT_)                                                         \
@@ -298,7 +298,7 @@ static int lm_pick(dim3 grid, size_t lds, hipStream_t stream, const LmArgs& a) {
     if (ndc <= 10) return lm_launch<WAVES_, NDT_, 10, SPLIT_>(grid, lds, stream, a);         \
     return lm_launch<WAVES_, NDT_, 22, SPLIT_>(grid, lds, stream, a);
     if (ndt <= 8) { LM_ROW(4, 8, 1) }
-    if (ndt <= 16) { LM_ROW(4, 16, 1) }
+    if (ndt <= 16) { LM_ROW(8, 16, 2) }
     LM_ROW(8, 32, 2)
 #undef LM_ROW
 }
