@@ -1,10 +1,10 @@
 // The attention over a shared latent (latent.hip) on MFMA, bfloat16, for the prompt portions and the single tokens of a step.
 //
 // Every head reads the same cached rows, so a block stages a run of 32 rows in LDS once, as they lie (for the scores) and
-// transposed (latent channels x rows, for the results), and each of its wavefronts works on a tile of 16 (token, head)
-// pairs of its own with them:
-//   a prompt tile  : 16 consecutive tokens of one portion; the block's four wavefronts take four heads;
-//   a single token : its heads, 16 a tile (a block's wavefronts take up to 64 heads); the token's visible rows are dealt in
+// transposed (latent channels x rows, for the results), and works on four tiles of 16 (token, head) pairs with them, one
+// wavefront a tile, or two where the latent has more than 128 channels (each with half of them):
+//   a prompt tile  : 16 consecutive tokens of one portion; the block's four tiles are four heads;
+//   a single token : its heads, 16 a tile (a block takes up to 64 heads); the token's visible rows are dealt in
 //                    chunks of one or more runs (aligned to absolute positions; how many runs follows from how far the
 //                    model lets a token see, not from the step) to blocks of their own, whose unnormalized results with
 //                    their maxima and sums are merged in chunk order: few tokens then fill the chip.
